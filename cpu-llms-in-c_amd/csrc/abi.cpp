@@ -1,0 +1,435 @@
+// The C ABI declared in include/mi355q.h: argument checking, device state,
+// host<->device staging and dispatch to the kernel launchers.
+#include "internal.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+namespace mi355q {
+
+void set_error(char *error, size_t capacity, const char *format, ...)
+{
+    if (error == nullptr || capacity == 0) return;
+    va_list args;
+    va_start(args, format);
+    vsnprintf(error, capacity, format, args);
+    va_end(args);
+}
+
+int fail_hip(hipError_t status, const char *what, char *error, size_t capacity)
+{
+    set_error(error, capacity, "%s: %s", what, hipGetErrorString(status));
+    (void)hipGetLastError();  // do not leave the error for the next call to trip over
+    return MI355Q_ERROR_RUNTIME;
+}
+
+int ensure_partials(mi355q_context *ctx, size_t bytes, size_t counters,
+                    char *error, size_t error_capacity)
+{
+    if (bytes > ctx->partials_bytes) {
+        MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before workspace growth");
+        if (ctx->partials) (void)hipFree(ctx->partials);
+        ctx->partials = nullptr;
+        ctx->partials_bytes = 0;
+        size_t want = bytes + bytes / 2;
+        MI355Q_HIP(hipMalloc((void **)&ctx->partials, want), "workspace allocation");
+        ctx->partials_bytes = want;
+    }
+    if (counters > ctx->counters_count) {
+        MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before counter growth");
+        if (ctx->counters) (void)hipFree(ctx->counters);
+        ctx->counters = nullptr;
+        ctx->counters_count = 0;
+        size_t want = counters * 2;
+        MI355Q_HIP(hipMalloc((void **)&ctx->counters, want * sizeof(uint32_t)),
+                   "counter allocation");
+        MI355Q_HIP(hipMemsetAsync(ctx->counters, 0, want * sizeof(uint32_t), ctx->stream),
+                   "counter clear");
+        ctx->counters_count = want;
+    }
+    return MI355Q_OK;
+}
+
+int ensure_stage(mi355q_context *ctx, int slot, size_t bytes, char *error,
+                 size_t error_capacity)
+{
+    if (bytes <= ctx->stage_bytes[slot]) return MI355Q_OK;
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before staging growth");
+    if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
+    ctx->stage[slot] = nullptr;
+    ctx->stage_bytes[slot] = 0;
+    size_t want = bytes + bytes / 2;
+    MI355Q_HIP(hipMalloc(&ctx->stage[slot], want), "staging allocation");
+    ctx->stage_bytes[slot] = want;
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" {
+
+int mi355q_context_create(int device, mi355q_context **out, char *error,
+                          size_t error_capacity)
+{
+    if (out == nullptr || device < 0) {
+        set_error(error, error_capacity, "context_create: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    *out = nullptr;
+    int count = 0;
+    MI355Q_HIP(hipGetDeviceCount(&count), "hipGetDeviceCount");
+    if (device >= count) {
+        set_error(error, error_capacity, "context_create: device %d of %d", device, count);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(device), "hipSetDevice");
+    mi355q_context *ctx = new (std::nothrow) mi355q_context();
+    if (ctx == nullptr) {
+        set_error(error, error_capacity, "context_create: out of host memory");
+        return MI355Q_ERROR_RUNTIME;
+    }
+    memset(ctx, 0, sizeof *ctx);
+    ctx->device = device;
+    hipError_t status = hipGetDeviceProperties(&ctx->props, device);
+    if (status == hipSuccess && strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
+        set_error(error, error_capacity, "context_create: device is %s, kernels are built for gfx950",
+                  ctx->props.gcnArchName);
+        delete ctx;
+        return MI355Q_ERROR_RUNTIME;
+    }
+    if (status == hipSuccess) status = hipStreamCreate(&ctx->stream);
+    if (status == hipSuccess) status = hipEventCreate(&ctx->timer_start);
+    if (status == hipSuccess) status = hipEventCreate(&ctx->timer_stop);
+    if (status != hipSuccess) {
+        int code = fail_hip(status, "context_create", error, error_capacity);
+        mi355q_context_destroy(ctx);
+        return code;
+    }
+    *out = ctx;
+    return MI355Q_OK;
+}
+
+void mi355q_context_destroy(mi355q_context *ctx)
+{
+    if (ctx == nullptr) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->partials) (void)hipFree(ctx->partials);
+    if (ctx->counters) (void)hipFree(ctx->counters);
+    for (int slot = 0; slot < 3; ++slot)
+        if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
+    if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
+    if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info, char *error,
+                        size_t error_capacity)
+{
+    if (ctx == nullptr || info == nullptr) {
+        set_error(error, error_capacity, "context_info: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    memset(info, 0, sizeof *info);
+    snprintf(info->name, sizeof info->name, "%s", ctx->props.name);
+    snprintf(info->arch, sizeof info->arch, "%s", ctx->props.gcnArchName);
+    info->compute_units = ctx->props.multiProcessorCount;
+    info->wavefront = ctx->props.warpSize;
+    info->hbm_bytes = ctx->props.totalGlobalMem;
+    info->lds_per_workgroup = ctx->props.sharedMemPerBlock;
+    info->clock_mhz = ctx->props.clockRate / 1000;
+    info->memory_clock_mhz = ctx->props.memoryClockRate / 1000;
+    info->memory_bus_bits = ctx->props.memoryBusWidth;
+    return MI355Q_OK;
+}
+
+int mi355q_sync(mi355q_context *ctx, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr) {
+        set_error(error, error_capacity, "sync: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return MI355Q_OK;
+}
+
+int mi355q_device_alloc(mi355q_context *ctx, size_t bytes, void **out, char *error,
+                        size_t error_capacity)
+{
+    if (ctx == nullptr || out == nullptr || bytes == 0) {
+        set_error(error, error_capacity, "device_alloc: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    *out = nullptr;
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    MI355Q_HIP(hipMalloc(out, bytes), "hipMalloc");
+    return MI355Q_OK;
+}
+
+int mi355q_device_free(mi355q_context *ctx, void *pointer, char *error,
+                       size_t error_capacity)
+{
+    if (ctx == nullptr) {
+        set_error(error, error_capacity, "device_free: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (pointer == nullptr) return MI355Q_OK;
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    MI355Q_HIP(hipFree(pointer), "hipFree");
+    return MI355Q_OK;
+}
+
+int mi355q_upload(mi355q_context *ctx, void *device_dst, const void *host_src,
+                  size_t bytes, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || device_dst == nullptr || host_src == nullptr) {
+        set_error(error, error_capacity, "upload: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (bytes == 0) return MI355Q_OK;
+    MI355Q_HIP(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, ctx->stream),
+               "upload");
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "upload sync");
+    return MI355Q_OK;
+}
+
+int mi355q_download(mi355q_context *ctx, void *host_dst, const void *device_src,
+                    size_t bytes, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || host_dst == nullptr || device_src == nullptr) {
+        set_error(error, error_capacity, "download: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (bytes == 0) return MI355Q_OK;
+    MI355Q_HIP(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, ctx->stream),
+               "download");
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "download sync");
+    return MI355Q_OK;
+}
+
+int mi355q_timer_begin(mi355q_context *ctx, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr) {
+        set_error(error, error_capacity, "timer_begin: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipEventRecord(ctx->timer_start, ctx->stream), "hipEventRecord");
+    ctx->timer_open = true;
+    return MI355Q_OK;
+}
+
+int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms, char *error,
+                     size_t error_capacity)
+{
+    if (ctx == nullptr || gpu_ms == nullptr || !ctx->timer_open) {
+        set_error(error, error_capacity, "timer_end: no timer_begin on this context");
+        return MI355Q_ERROR_INVALID;
+    }
+    ctx->timer_open = false;
+    MI355Q_HIP(hipEventRecord(ctx->timer_stop, ctx->stream), "hipEventRecord");
+    MI355Q_HIP(hipEventSynchronize(ctx->timer_stop), "hipEventSynchronize");
+    float ms = 0.0f;
+    MI355Q_HIP(hipEventElapsedTime(&ms, ctx->timer_start, ctx->timer_stop),
+               "hipEventElapsedTime");
+    *gpu_ms = (double)ms;
+    return MI355Q_OK;
+}
+
+// ---- affine Q4 ---------------------------------------------------------------
+
+int mi355q_q4_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
+                             const void *meta_b, uint32_t N, uint32_t K, int meta_kind,
+                             uint32_t flags, mi355q_q4_weight **out, char *error,
+                             size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    if (ctx == nullptr || out == nullptr || quants == nullptr || meta_a == nullptr) {
+        set_error(error, error_capacity, "q4_weight_prepare: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (meta_kind != MI355Q_META_F16_INTERLEAVED && meta_kind != MI355Q_META_BF16_PLANES) {
+        set_error(error, error_capacity, "q4_weight_prepare: unknown metadata kind %d", meta_kind);
+        return MI355Q_ERROR_INVALID;
+    }
+    if (meta_kind == MI355Q_META_BF16_PLANES && meta_b == nullptr) {
+        set_error(error, error_capacity, "q4_weight_prepare: bf16 planes need a bias plane");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (N == 0 || K == 0 || K % 64u != 0) {
+        set_error(error, error_capacity,
+                  "q4_weight_prepare: shape %u x %u (columns must be a non-zero multiple of 64)",
+                  N, K);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+
+    mi355q_q4_weight *weight = new (std::nothrow) mi355q_q4_weight();
+    if (weight == nullptr) {
+        set_error(error, error_capacity, "q4_weight_prepare: out of host memory");
+        return MI355Q_ERROR_RUNTIME;
+    }
+    memset(weight, 0, sizeof *weight);
+    weight->ctx = ctx;
+    Q4Device &dev = weight->dev;
+    dev.N = N;
+    dev.K = K;
+    dev.NT = (N + kTileRows - 1) / kTileRows;
+    dev.T = (K + kStepColumns - 1) / kStepColumns;
+    dev.meta_kind = meta_kind;
+    const size_t groups = (size_t)N * (K / 64u);
+    const size_t code_bytes = (size_t)N * (K / 2u);
+    const size_t meta_bytes = groups * 4u;
+    weight->image_bytes = code_bytes + meta_bytes;
+
+    const bool on_device = (flags & MI355Q_SOURCE_DEVICE) != 0;
+    void *staging = nullptr;
+    const uint32_t *src_codes = (const uint32_t *)quants;
+    const uint16_t *src_a = (const uint16_t *)meta_a;
+    const uint16_t *src_b = (const uint16_t *)meta_b;
+    hipError_t status = hipSuccess;
+    const char *what = "q4_weight_prepare";
+    do {
+        what = "weight allocation";
+        status = hipMalloc((void **)&dev.codes, (size_t)dev.NT * dev.T * 64u * sizeof(uint4));
+        if (status != hipSuccess) break;
+        status = hipMalloc((void **)&dev.meta, (size_t)dev.NT * dev.T * 16u * sizeof(uint2));
+        if (status != hipSuccess) break;
+        if (!on_device) {
+            what = "image upload";
+            status = hipMalloc(&staging, code_bytes + meta_bytes);
+            if (status != hipSuccess) break;
+            char *base = (char *)staging;
+            status = hipMemcpyAsync(base, quants, code_bytes, hipMemcpyHostToDevice, ctx->stream);
+            if (status != hipSuccess) break;
+            src_codes = (const uint32_t *)base;
+            if (meta_kind == MI355Q_META_F16_INTERLEAVED) {
+                status = hipMemcpyAsync(base + code_bytes, meta_a, meta_bytes,
+                                        hipMemcpyHostToDevice, ctx->stream);
+                src_a = (const uint16_t *)(base + code_bytes);
+                src_b = nullptr;
+            } else {
+                status = hipMemcpyAsync(base + code_bytes, meta_a, meta_bytes / 2,
+                                        hipMemcpyHostToDevice, ctx->stream);
+                if (status != hipSuccess) break;
+                status = hipMemcpyAsync(base + code_bytes + meta_bytes / 2, meta_b,
+                                        meta_bytes / 2, hipMemcpyHostToDevice, ctx->stream);
+                src_a = (const uint16_t *)(base + code_bytes);
+                src_b = (const uint16_t *)(base + code_bytes + meta_bytes / 2);
+            }
+            if (status != hipSuccess) break;
+        }
+        what = "re-tiling";
+        status = q4_repack_launch(src_codes, src_a, src_b, dev, ctx->stream);
+        if (status != hipSuccess) break;
+        status = hipStreamSynchronize(ctx->stream);
+    } while (false);
+    if (staging) (void)hipFree(staging);
+    if (status != hipSuccess) {
+        int code = fail_hip(status, what, error, error_capacity);
+        mi355q_q4_weight_destroy(weight);
+        return code;
+    }
+    *out = weight;
+    return MI355Q_OK;
+}
+
+void mi355q_q4_weight_destroy(mi355q_q4_weight *weight)
+{
+    if (weight == nullptr) return;
+    if (weight->ctx) {
+        (void)hipSetDevice(weight->ctx->device);
+        (void)hipStreamSynchronize(weight->ctx->stream);
+    }
+    if (weight->dev.codes) (void)hipFree(weight->dev.codes);
+    if (weight->dev.meta) (void)hipFree(weight->dev.meta);
+    delete weight;
+}
+
+size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight)
+{
+    return weight ? weight->image_bytes : 0;
+}
+
+int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const void *x,
+                     int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,
+                     int residual_dtype, uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || x == nullptr || y == nullptr) {
+        set_error(error, error_capacity, "q4_linear: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "q4_linear: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (M == 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype) ||
+        (residual != nullptr && !dtype_valid(residual_dtype))) {
+        set_error(error, error_capacity, "q4_linear: M=%u x_dtype=%d y_dtype=%d residual_dtype=%d",
+                  M, x_dtype, y_dtype, residual_dtype);
+        return MI355Q_ERROR_INVALID;
+    }
+    const bool x_dev = flags & MI355Q_X_DEVICE, y_dev = flags & MI355Q_Y_DEVICE;
+    const bool r_dev = residual == nullptr || (flags & MI355Q_RESIDUAL_DEVICE);
+    if ((flags & MI355Q_ASYNC) && !(x_dev && y_dev && r_dev)) {
+        set_error(error, error_capacity, "q4_linear: ASYNC needs device pointers throughout");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (x_dev && ((uintptr_t)x & 15u) != 0) {
+        set_error(error, error_capacity, "q4_linear: device x must be 16-byte aligned");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const Q4Device &dev = weight->dev;
+    const size_t x_bytes = (size_t)M * dev.K * dtype_bytes(x_dtype);
+    const size_t y_bytes = (size_t)M * dev.N * dtype_bytes(y_dtype);
+    const size_t r_bytes = residual ? (size_t)M * dev.N * dtype_bytes(residual_dtype) : 0;
+
+    Q4LinearArgs args;
+    args.x = x;
+    args.x_dtype = x_dtype;
+    args.M = M;
+    args.y = y;
+    args.y_dtype = y_dtype;
+    args.residual = residual;
+    args.residual_dtype = residual_dtype;
+    int status;
+    if (!x_dev) {
+        if ((status = ensure_stage(ctx, 0, x_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[0], x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "activation upload");
+        args.x = ctx->stage[0];
+    }
+    if (!y_dev) {
+        if ((status = ensure_stage(ctx, 1, y_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        args.y = ctx->stage[1];
+    }
+    if (!r_dev) {
+        if ((status = ensure_stage(ctx, 2, r_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[2], residual, r_bytes, hipMemcpyHostToDevice,
+                                  ctx->stream),
+                   "residual upload");
+        args.residual = ctx->stage[2];
+    }
+
+    const uint32_t stream_rows = x_dtype == MI355Q_F32 ? 2u * M : M;
+    if (stream_rows <= 16u) {
+        status = q4_stream_linear(ctx, dev, args, error, error_capacity);
+    } else {
+        set_error(error, error_capacity, "q4_linear: M=%u is not supported yet", M);
+        status = MI355Q_ERROR_INVALID;
+    }
+    if (status != MI355Q_OK) return status;
+
+    if (!y_dev)
+        MI355Q_HIP(hipMemcpyAsync(y, ctx->stage[1], y_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                   "output download");
+    if (!(flags & MI355Q_ASYNC))
+        MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear sync");
+    return MI355Q_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+// Internal declarations shared by the C-ABI layer and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "mi355q.h"
+
+namespace mi355q {
+
+// ---- device weight layout -------------------------------------------------
+// An affine-Q4 weight is kept in HBM as "stream tiles": 16 output rows x 128
+// input columns = 1 KiB of codes, stored so that lane l of a wavefront reads
+// its 16 bytes at offset 16*l.  Lane l = (row r = l % 16, quarter kq = l / 16)
+// holds four dwords; dword d is the row's original little-endian code word
+// number 4*d + kq of the 16 words in the 128-column step, i.e. columns
+// 32*d + 8*kq .. +7.  One 16x16x32 MFMA therefore consumes dword d of every
+// lane and covers the contiguous columns 32*d .. 32*d+31 (half a group).
+// Metadata: per (tile, step, row) eight bytes = {scale,bias} of group 2*step
+// then of group 2*step+1, 16-bit fields in the image's own encoding.
+// Rows beyond N and columns beyond K are padded with zero codes and zero
+// metadata, which contribute exactly 0.
+constexpr uint32_t kTileRows = 16;
+constexpr uint32_t kStepColumns = 128;
+
+struct Q4Device {
+    uint4 *codes;   // [NT][T][64]
+    uint2 *meta;    // [NT][T][16]
+    uint32_t N, K;  // logical shape
+    uint32_t NT, T; // tiles of 16 rows, steps of 128 columns
+    int meta_kind;
+};
+
+}  // namespace mi355q
+
+struct mi355q_context {
+    int device;
+    hipStream_t stream;
+    hipEvent_t timer_start, timer_stop;
+    bool timer_open;
+    hipDeviceProp_t props;
+    // split-K workspace: fp32 partial sums and one arrival counter per
+    // workgroup column; counters are zero between calls.
+    float *partials;
+    size_t partials_bytes;
+    uint32_t *counters;
+    size_t counters_count;
+    // staging for host-pointer activations / outputs
+    void *stage[3];
+    size_t stage_bytes[3];
+};
+
+struct mi355q_q4_weight {
+    mi355q_context *ctx;
+    mi355q::Q4Device dev;
+    size_t image_bytes;
+};
+
+namespace mi355q {
+
+void set_error(char *error, size_t capacity, const char *format, ...);
+int fail_hip(hipError_t status, const char *what, char *error, size_t capacity);
+
+#define MI355Q_HIP(call, what)                                              \
+    do {                                                                    \
+        hipError_t status_ = (call);                                        \
+        if (status_ != hipSuccess)                                          \
+            return ::mi355q::fail_hip(status_, what, error, error_capacity); \
+    } while (0)
+
+int ensure_partials(mi355q_context *ctx, size_t bytes, size_t counters,
+                    char *error, size_t error_capacity);
+int ensure_stage(mi355q_context *ctx, int slot, size_t bytes,
+                 char *error, size_t error_capacity);
+
+inline size_t dtype_bytes(int dtype) { return dtype == MI355Q_F32 ? 4u : 2u; }
+inline bool dtype_valid(int dtype) {
+    return dtype == MI355Q_F16 || dtype == MI355Q_F32 || dtype == MI355Q_BF16;
+}
+
+// q4_layout.hip
+hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
+                            const uint16_t *meta_b, const Q4Device &dst,
+                            hipStream_t stream);
+
+// q4_stream.hip
+struct Q4LinearArgs {
+    const void *x;
+    int x_dtype;
+    uint32_t M;
+    void *y;
+    int y_dtype;
+    const void *residual;
+    int residual_dtype;
+};
+int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
+                     char *error, size_t error_capacity);
+
+}  // namespace mi355q

@@ -1,0 +1,90 @@
+// Re-tiles an affine-Q4 image (row-major code plane + metadata plane(s)) into
+// the stream-tile order described in internal.h.  One-time work at prepare.
+#include "internal.h"
+
+namespace mi355q {
+
+// One thread per destination uint4.  src_words is the image's code plane seen
+// as little-endian uint32 [N][K/8] (compiler/qwen3.8-27b/apple-m3-pro/
+// qwen38_m3_pack.c:618-637 describes the same bytes as U32 [N, K/8]).
+__global__ void __launch_bounds__(256)
+q4_repack_codes_kernel(const uint32_t *__restrict__ src_words, uint4 *__restrict__ dst,
+                       uint32_t N, uint32_t K, uint32_t NT, uint32_t T)
+{
+    uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t total = (uint64_t)NT * T * 64u;
+    if (index >= total) return;
+    uint32_t lane = (uint32_t)(index & 63u);
+    uint64_t tile_step = index >> 6;
+    uint32_t step = (uint32_t)(tile_step % T);
+    uint32_t tile = (uint32_t)(tile_step / T);
+    uint32_t row = tile * kTileRows + (lane & 15u);
+    uint32_t kq = lane >> 4;
+    uint32_t words_per_row = K / 8u;
+    uint32_t out[4];
+#pragma unroll
+    for (uint32_t d = 0; d < 4; ++d) {
+        uint32_t word = step * 16u + 4u * d + kq;
+        out[d] = (row < N && word < words_per_row)
+                     ? src_words[(uint64_t)row * words_per_row + word]
+                     : 0u;
+    }
+    dst[index] = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+// One thread per (tile, step, row).  BF16 planes are interleaved here so the
+// kernels read one 8-byte record per step whatever the image kind.
+__global__ void __launch_bounds__(256)
+q4_repack_meta_kernel(const uint16_t *__restrict__ meta_a,
+                      const uint16_t *__restrict__ meta_b, int meta_kind,
+                      uint2 *__restrict__ dst, uint32_t N, uint32_t K, uint32_t NT,
+                      uint32_t T)
+{
+    uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t total = (uint64_t)NT * T * 16u;
+    if (index >= total) return;
+    uint32_t r = (uint32_t)(index & 15u);
+    uint64_t tile_step = index >> 4;
+    uint32_t step = (uint32_t)(tile_step % T);
+    uint32_t tile = (uint32_t)(tile_step / T);
+    uint32_t row = tile * kTileRows + r;
+    uint32_t groups = K / 64u;
+    uint32_t out[2];
+#pragma unroll
+    for (uint32_t h = 0; h < 2; ++h) {
+        uint32_t group = 2u * step + h;
+        uint32_t value = 0u;
+        if (row < N && group < groups) {
+            uint64_t block = (uint64_t)row * groups + group;
+            uint32_t scale, bias;
+            if (meta_kind == MI355Q_META_F16_INTERLEAVED) {
+                scale = meta_a[2u * block];
+                bias = meta_a[2u * block + 1u];
+            } else {
+                scale = meta_a[block];
+                bias = meta_b[block];
+            }
+            value = scale | (bias << 16);
+        }
+        out[h] = value;
+    }
+    dst[index] = make_uint2(out[0], out[1]);
+}
+
+hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
+                            const uint16_t *meta_b, const Q4Device &dst,
+                            hipStream_t stream)
+{
+    uint64_t code_items = (uint64_t)dst.NT * dst.T * 64u;
+    uint64_t meta_items = (uint64_t)dst.NT * dst.T * 16u;
+    uint32_t code_blocks = (uint32_t)((code_items + 255u) / 256u);
+    uint32_t meta_blocks = (uint32_t)((meta_items + 255u) / 256u);
+    hipLaunchKernelGGL(q4_repack_codes_kernel, dim3(code_blocks), dim3(256), 0, stream,
+                       codes_src, dst.codes, dst.N, dst.K, dst.NT, dst.T);
+    hipLaunchKernelGGL(q4_repack_meta_kernel, dim3(meta_blocks), dim3(256), 0, stream,
+                       meta_a, meta_b, dst.meta_kind, dst.meta, dst.N, dst.K, dst.NT,
+                       dst.T);
+    return hipGetLastError();
+}
+
+}  // namespace mi355q

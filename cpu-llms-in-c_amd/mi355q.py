@@ -1,0 +1,259 @@
+"""ctypes binding of libmi355q.so (include/mi355q.h, include/mi355q_synth.h).
+
+Used by the tests, the smoke check and bench.py.  It only loads the library
+that `make -C cpu-llms-in-c_amd/csrc` (or __graft_entry__.build) has built in
+cpu-llms-in-c_amd/lib; there is no fallback of any kind: a missing library or a
+missing GPU raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+
+import numpy as np
+
+PACKAGE_DIR = Path(__file__).resolve().parent
+LIBRARY_PATH = PACKAGE_DIR / "lib" / "libmi355q.so"
+
+OK, ERROR_RUNTIME, ERROR_INVALID = 0, 1, 2
+F16, F32, BF16 = 0, 1, 2
+META_F16_INTERLEAVED, META_BF16_PLANES = 0, 1
+X_DEVICE, Y_DEVICE, RESIDUAL_DEVICE, ASYNC, SOURCE_DEVICE = 1, 2, 4, 8, 16
+
+_c = ctypes
+_u32, _u64, _sz, _int = _c.c_uint32, _c.c_uint64, _c.c_size_t, _c.c_int
+_vp, _cp = _c.c_void_p, _c.c_char_p
+_err = (_c.c_char_p, _c.c_size_t)
+
+
+class DeviceInfo(_c.Structure):
+    _fields_ = [
+        ("name", _c.c_char * 128),
+        ("arch", _c.c_char * 32),
+        ("compute_units", _int),
+        ("wavefront", _int),
+        ("hbm_bytes", _sz),
+        ("lds_per_workgroup", _sz),
+        ("clock_mhz", _int),
+        ("memory_clock_mhz", _int),
+        ("memory_bus_bits", _int),
+    ]
+
+
+# name -> (restype, argtypes): every symbol the two headers declare
+SIGNATURES = {
+    "mi355q_context_create": (_int, [_int, _c.POINTER(_vp), *_err]),
+    "mi355q_context_destroy": (None, [_vp]),
+    "mi355q_context_info": (_int, [_vp, _c.POINTER(DeviceInfo), *_err]),
+    "mi355q_sync": (_int, [_vp, *_err]),
+    "mi355q_device_alloc": (_int, [_vp, _sz, _c.POINTER(_vp), *_err]),
+    "mi355q_device_free": (_int, [_vp, _vp, *_err]),
+    "mi355q_upload": (_int, [_vp, _vp, _vp, _sz, *_err]),
+    "mi355q_download": (_int, [_vp, _vp, _vp, _sz, *_err]),
+    "mi355q_timer_begin": (_int, [_vp, *_err]),
+    "mi355q_timer_end": (_int, [_vp, _c.POINTER(_c.c_double), *_err]),
+    "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
+                                        _c.POINTER(_vp), *_err]),
+    "mi355q_q4_weight_destroy": (None, [_vp]),
+    "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
+    "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
+    "mi355q_synth_normal_f32": (None, [_u64, _c.c_float, _sz, _vp]),
+    "mi355q_synth_normal_f16": (None, [_u64, _c.c_float, _sz, _vp]),
+    "mi355q_quantize_q4_affine": (_int, [_vp, _u32, _u32, _int, _vp, _vp, _vp]),
+    "mi355q_synth_q4_affine": (_int, [_u64, _c.c_float, _u32, _u32, _int, _vp, _vp, _vp]),
+    "mi355q_quantize_w8_rows": (_int, [_vp, _u32, _u32, _vp]),
+    "mi355q_synth_w8_rows": (_int, [_u64, _c.c_float, _u32, _u32, _vp]),
+}
+
+_library = None
+
+
+class Mi355qError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"mi355q status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+def library() -> ctypes.CDLL:
+    """Loads libmi355q.so (once) and types every exported function."""
+    global _library
+    if _library is None:
+        if not LIBRARY_PATH.exists():
+            raise FileNotFoundError(
+                f"{LIBRARY_PATH} is not built; run `make -C {PACKAGE_DIR / 'csrc'}`")
+        lib = ctypes.CDLL(os.fspath(LIBRARY_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            function = getattr(lib, name)
+            function.restype = restype
+            function.argtypes = argtypes
+        _library = lib
+    return _library
+
+
+def _ptr(array):
+    if array is None:
+        return None
+    if isinstance(array, (int, ctypes.c_void_p)):
+        return array
+    assert array.flags["C_CONTIGUOUS"]
+    return array.ctypes.data_as(ctypes.c_void_p)
+
+
+def _call(function, *args):
+    error = ctypes.create_string_buffer(512)
+    status = function(*args, error, len(error))
+    if status != OK:
+        raise Mi355qError(status, error.value.decode(errors="replace"))
+
+
+_NP_DTYPE = {F16: np.float16, F32: np.float32, BF16: np.uint16}
+
+
+class Q4Weight:
+    def __init__(self, context: "Context", handle, N: int, K: int):
+        self.context, self.handle, self.N, self.K = context, handle, N, K
+
+    @property
+    def image_bytes(self) -> int:
+        return library().mi355q_q4_weight_image_bytes(self.handle)
+
+    def destroy(self):
+        if self.handle:
+            library().mi355q_q4_weight_destroy(self.handle)
+            self.handle = None
+
+
+class Context:
+    """One engine context (one HIP stream) on one GPU."""
+
+    def __init__(self, device: int = 0):
+        self.lib = library()
+        handle = ctypes.c_void_p()
+        _call(self.lib.mi355q_context_create, device, ctypes.byref(handle))
+        self.handle = handle
+
+    def close(self):
+        if self.handle:
+            self.lib.mi355q_context_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def info(self) -> DeviceInfo:
+        info = DeviceInfo()
+        _call(self.lib.mi355q_context_info, self.handle, ctypes.byref(info))
+        return info
+
+    def sync(self):
+        _call(self.lib.mi355q_sync, self.handle)
+
+    def alloc(self, nbytes: int) -> int:
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_device_alloc, self.handle, nbytes, ctypes.byref(out))
+        return out.value
+
+    def free(self, pointer: int):
+        _call(self.lib.mi355q_device_free, self.handle, pointer)
+
+    def upload(self, pointer: int, array: np.ndarray):
+        array = np.ascontiguousarray(array)
+        _call(self.lib.mi355q_upload, self.handle, pointer, _ptr(array), array.nbytes)
+
+    def to_device(self, array: np.ndarray) -> int:
+        pointer = self.alloc(max(array.nbytes, 16))
+        self.upload(pointer, array)
+        return pointer
+
+    def download(self, pointer: int, shape, dtype) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        _call(self.lib.mi355q_download, self.handle, _ptr(out), pointer, out.nbytes)
+        return out
+
+    def timer_begin(self):
+        _call(self.lib.mi355q_timer_begin, self.handle)
+
+    def timer_end(self) -> float:
+        ms = ctypes.c_double()
+        _call(self.lib.mi355q_timer_end, self.handle, ctypes.byref(ms))
+        return ms.value
+
+    # ---- affine Q4 ----
+    def q4_prepare(self, quants, meta_a, meta_b, N: int, K: int, meta_kind: int,
+                   flags: int = 0) -> Q4Weight:
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_q4_weight_prepare, self.handle, _ptr(quants), _ptr(meta_a),
+              _ptr(meta_b), N, K, meta_kind, flags, ctypes.byref(out))
+        return Q4Weight(self, out, N, K)
+
+    def q4_linear(self, weight: Q4Weight, x: np.ndarray, x_dtype: int, y_dtype: int = F32,
+                  residual: np.ndarray | None = None, residual_dtype: int = F32) -> np.ndarray:
+        """Host-array convenience form: x [M][K] -> y [M][N]."""
+        x = np.ascontiguousarray(x)
+        M = x.shape[0]
+        y = np.empty((M, weight.N), dtype=_NP_DTYPE[y_dtype])
+        _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, _ptr(x), x_dtype, M,
+              _ptr(y), y_dtype, _ptr(residual), residual_dtype, 0)
+        return y
+
+    def q4_linear_device(self, weight: Q4Weight, x_ptr: int, x_dtype: int, M: int, y_ptr: int,
+                         y_dtype: int, residual_ptr: int | None = None,
+                         residual_dtype: int = F32, asynchronous: bool = True):
+        flags = X_DEVICE | Y_DEVICE | RESIDUAL_DEVICE | (ASYNC if asynchronous else 0)
+        _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, x_ptr, x_dtype, M, y_ptr,
+              y_dtype, residual_ptr, residual_dtype, flags)
+
+
+# ---- synthetic inputs (host side) ------------------------------------------
+
+def synth_normal_f32(seed: int, sigma: float, count: int) -> np.ndarray:
+    out = np.empty(count, dtype=np.float32)
+    library().mi355q_synth_normal_f32(seed, sigma, count, _ptr(out))
+    return out
+
+
+def synth_normal_f16(seed: int, sigma: float, count: int) -> np.ndarray:
+    out = np.empty(count, dtype=np.float16)
+    library().mi355q_synth_normal_f16(seed, sigma, count, _ptr(out))
+    return out
+
+
+def _q4_planes(N: int, K: int, meta_kind: int):
+    groups = N * (K // 64)
+    quants = np.empty(groups * 32, dtype=np.uint8)
+    if meta_kind == META_F16_INTERLEAVED:
+        return quants, np.empty(groups * 2, dtype=np.uint16), None
+    return quants, np.empty(groups, dtype=np.uint16), np.empty(groups, dtype=np.uint16)
+
+
+def quantize_q4_affine(w: np.ndarray, meta_kind: int):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    N, K = w.shape
+    quants, meta_a, meta_b = _q4_planes(N, K, meta_kind)
+    status = library().mi355q_quantize_q4_affine(_ptr(w), N, K, meta_kind, _ptr(quants),
+                                                 _ptr(meta_a), _ptr(meta_b))
+    if status != OK:
+        raise Mi355qError(status, "quantize_q4_affine: bad shape")
+    return quants, meta_a, meta_b
+
+
+def synth_q4_affine(seed: int, sigma: float, N: int, K: int, meta_kind: int):
+    quants, meta_a, meta_b = _q4_planes(N, K, meta_kind)
+    status = library().mi355q_synth_q4_affine(seed, sigma, N, K, meta_kind, _ptr(quants),
+                                              _ptr(meta_a), _ptr(meta_b))
+    if status != OK:
+        raise Mi355qError(status, "synth_q4_affine: bad shape")
+    return quants, meta_a, meta_b
+
+
+def synth_w8_rows(seed: int, sigma: float, N: int, K: int) -> np.ndarray:
+    rows = np.empty(N * (4 + K), dtype=np.uint8)
+    status = library().mi355q_synth_w8_rows(seed, sigma, N, K, _ptr(rows))
+    if status != OK:
+        raise Mi355qError(status, "synth_w8_rows: bad shape")
+    return rows

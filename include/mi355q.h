@@ -1,0 +1,153 @@
+/* mi355q — quantized-linear engine for AMD Instinct MI355X (gfx950).
+ *
+ * C ABI of the drop-in replacement for the quantized linear / matmul calls of
+ * the llm-in-c C runtimes.  Plain pointers and sizes only.  Every entry point
+ * returns an int status and, on failure, writes a message into the caller's
+ * buffer (NULL / zero capacity is tolerated) — the convention of the
+ * reference's C entry points (models/qwen3.8-27b/targets/apple-m3-pro/
+ * qwen38_m3.m:35-41,342-345; models/minimax-h3/targets/apple-m3-pro/
+ * minimax_h3_m3_gemm.m:309-315: 0 ok, 1 device/runtime failure, 2 invalid
+ * argument).  Nothing aborts.
+ *
+ * Weight images are consumed in the byte layouts the reference's packers
+ * write; `*_weight_prepare` uploads them once into HBM (in a tiled order the
+ * kernels stream) and the handle is then used for any number of calls —
+ * the prepare-once / run-many shape of the reference's operators
+ * (models/whisper-large-v3-turbo/targets/rk3588/native/opencl_w4a16.h:93-133;
+ * minimax_h3_m3_gemm.m:338-346).
+ *
+ * Threading: one context owns one HIP stream and one workspace and permits
+ * one call in flight (as the reference's model handle does,
+ * qwen38_m3_decode.h:73-75).  Distinct contexts are independent.
+ */
+#ifndef MI355Q_H
+#define MI355Q_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mi355q_context mi355q_context;
+typedef struct mi355q_q4_weight mi355q_q4_weight;
+typedef struct mi355q_w8a8_weight mi355q_w8a8_weight;
+
+enum {
+    MI355Q_OK = 0,
+    MI355Q_ERROR_RUNTIME = 1,
+    MI355Q_ERROR_INVALID = 2
+};
+
+/* element types of activations, outputs and residuals */
+enum {
+    MI355Q_F16 = 0,
+    MI355Q_F32 = 1,
+    MI355Q_BF16 = 2
+};
+
+/* affine-Q4 group-64 metadata layouts */
+enum {
+    /* meta[N][K/64] of {uint16 fp16 scale, uint16 fp16 bias}: the Q38 image's
+     * metadata plane (qwen38_m3.m:19-33; qwen38_m3_image.h:40-51) */
+    MI355Q_META_F16_INTERLEAVED = 0,
+    /* scales[N][K/64] and biases[N][K/64], bf16: the MLX source planes
+     * (compiler/minimax-h3/apple-m3-pro/minimax_h3_q4_layer.h:14-24;
+     * qwen38_m3_pack.c:618-637) */
+    MI355Q_META_BF16_PLANES = 1
+};
+
+/* flags */
+enum {
+    MI355Q_X_DEVICE = 1u << 0,        /* x is a device pointer */
+    MI355Q_Y_DEVICE = 1u << 1,        /* y is a device pointer */
+    MI355Q_RESIDUAL_DEVICE = 1u << 2, /* residual is a device pointer */
+    MI355Q_ASYNC = 1u << 3,           /* do not wait; all pointers must be device */
+    MI355Q_SOURCE_DEVICE = 1u << 4    /* prepare: image pointers are device pointers */
+};
+
+typedef struct {
+    char name[128];
+    char arch[32];
+    int compute_units;
+    int wavefront;
+    size_t hbm_bytes;
+    size_t lds_per_workgroup;
+    int clock_mhz;
+    int memory_clock_mhz;
+    int memory_bus_bits;
+} mi355q_device_info;
+
+/* ---- context ---------------------------------------------------------------
+ * The opaque handle that owns device state, as qwen38_m3_model / the Metal
+ * device+queue do in the reference (qwen38_m3_decode.h:62-75). */
+int mi355q_context_create(int device, mi355q_context **out,
+                          char *error, size_t error_capacity);
+void mi355q_context_destroy(mi355q_context *ctx);
+int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
+                        char *error, size_t error_capacity);
+/* Waits for everything queued on the context's stream
+ * (the reference's waitUntilCompleted, qwen38_m3_decode.m:1701-1716). */
+int mi355q_sync(mi355q_context *ctx, char *error, size_t error_capacity);
+
+/* Device buffers for callers that keep activations resident between calls
+ * (the reference's MTLBuffer allocations, qwen38_m3.m:523-552). */
+int mi355q_device_alloc(mi355q_context *ctx, size_t bytes, void **out,
+                        char *error, size_t error_capacity);
+int mi355q_device_free(mi355q_context *ctx, void *pointer,
+                       char *error, size_t error_capacity);
+int mi355q_upload(mi355q_context *ctx, void *device_dst, const void *host_src,
+                  size_t bytes, char *error, size_t error_capacity);
+int mi355q_download(mi355q_context *ctx, void *host_dst, const void *device_src,
+                    size_t bytes, char *error, size_t error_capacity);
+
+/* GPU time of the work queued between the two calls, from HIP events on the
+ * context's stream — the `double *gpu_ms` the reference's projection call
+ * reports (minimax_h3_m3_gemm.h:58-66; GPUEndTime-GPUStartTime,
+ * qwen38_m3_decode.m:1217-1283). */
+int mi355q_timer_begin(mi355q_context *ctx, char *error, size_t error_capacity);
+int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms,
+                     char *error, size_t error_capacity);
+
+/* ---- affine Q4, group 64: w[n][k] = scale[n][k/64] * q[n][k] + bias[n][k/64]
+ *
+ * quants: [N][K/64][32] bytes, element k of a row in byte k/2, even k in the
+ *         low nibble (== little-endian uint32 [N][K/8], element k%8 at bits
+ *         4*(k%8)) — qwen38_m3.m:113-116; minimax_h3_attention.metal:246-255.
+ * meta_a / meta_b: per `meta_kind`; meta_b is NULL for the interleaved kind.
+ * K must be a non-zero multiple of 64 (minimax_h3_m3_gemm.m:309-315 rejects
+ * anything else with status 2); N is any non-zero row count.
+ * Replaces: the image-to-buffer step of qwen38_m3.m:523-552 and
+ * minimax_h3_m3_gemm.m:338-346. */
+int mi355q_q4_weight_prepare(mi355q_context *ctx,
+                             const void *quants, const void *meta_a,
+                             const void *meta_b, uint32_t N, uint32_t K,
+                             int meta_kind, uint32_t flags,
+                             mi355q_q4_weight **out,
+                             char *error, size_t error_capacity);
+void mi355q_q4_weight_destroy(mi355q_q4_weight *weight);
+/* Bytes of the original image this weight stands for: N*K/2 + N*(K/64)*4. */
+size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight);
+
+/* y[m][n] = sum_k w[n][k] * x[m][k]  (+ residual[m][n] when residual != NULL)
+ *
+ * x: [M][K] of x_dtype (F16, F32 or BF16); y: [M][N] of y_dtype; residual:
+ * [M][N] of residual_dtype.  The weight is evaluated as scale*q + bias without
+ * rounding for M <= 16 (fp32 accumulation throughout); for larger M the weight
+ * is rounded to fp16 before an fp16 matrix multiply with fp32 accumulation.
+ * Replaces: cpu_row_dot / qwen38_q4_matvec (qwen38_m3.m:102-121;
+ * qwen38_q4.metal:111-127), qwen38_q4_down_residual (qwen38_q4.metal:163-191),
+ * the batched qwen38_prefill_q4_gemm_f16* family (qwen38_prefill.metal:144-248,
+ * 797-1502) and minimax_h3_m3_run_q4_projection_bf16 (minimax_h3_m3_gemm.h:58-66). */
+int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight,
+                     const void *x, int x_dtype, uint32_t M,
+                     void *y, int y_dtype,
+                     const void *residual, int residual_dtype,
+                     uint32_t flags, char *error, size_t error_capacity);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

@@ -1,0 +1,120 @@
+"""GPU parity of the weight-streaming affine-Q4 linear (1..16 activation rows)
+against the CPU oracle, through the C ABI.
+
+Gate (Q4, fp32 accumulation): max_i |y_i - ref_i| / max(|ref_i|, 1e-2*rms(ref)) <= 1e-3,
+where ref is the oracle's exact-weight, double-accumulated result
+(reference semantics: qwen38_m3.m:102-121, weights not rounded).
+"""
+import numpy as np
+import pytest
+
+from conftest import bf16_bits, q4_relative_error
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1e-3
+
+
+def make_x(engine, seed, M, K, x_dtype):
+    rows = [engine.synth_normal_f32(seed + 1000 * m, 1.0, K) for m in range(M)]
+    x32 = np.stack(rows)
+    if x_dtype == engine.F16:
+        return x32.astype(np.float16)
+    if x_dtype == engine.BF16:
+        return bf16_bits(x32)
+    return x32
+
+
+def run_case(engine, oracle, gpu, N, K, M, meta_kind, x_dtype, y_dtype, seed=7, residual=False):
+    quants, meta_a, meta_b = engine.synth_q4_affine(seed, 0.02, N, K, meta_kind)
+    x = make_x(engine, seed + 1, M, K, x_dtype)
+    res = None
+    if residual:
+        res = engine.synth_normal_f32(seed + 2, 1.0, M * N).reshape(M, N)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, meta_kind)
+    try:
+        print(f"case N={N} K={K} M={M} meta={meta_kind} x={x_dtype} y={y_dtype} res={residual}",
+              flush=True)
+        y = gpu.q4_linear(weight, x, x_dtype, y_dtype, res, engine.F32)
+    finally:
+        weight.destroy()
+    ref = oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_dtype, M)
+    if residual:
+        ref = ref + res.astype(np.float64)
+    if y_dtype == engine.BF16:
+        y = (y.astype(np.uint32) << 16).view(np.float32)
+        tolerance = 2.0 ** -8  # bf16 output rounding dominates
+    else:
+        tolerance = TOLERANCE
+    error = q4_relative_error(y, ref)
+    assert np.all(np.isfinite(np.asarray(y, dtype=np.float64)))
+    assert error <= tolerance, f"relative error {error:.3e}"
+    return error
+
+
+def test_config1_gemv_fp16(engine, oracle, gpu):
+    """BASELINE config 1: K=1024, N=3584, M=1, fp16 scale/bias, fp16 x, fp16 y."""
+    run_case(engine, oracle, gpu, 3584, 1024, 1, engine.META_F16_INTERLEAVED, engine.F16, engine.F16)
+
+
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 64), (100, 192), (33, 1024), (257, 1088),
+                                 (16480, 512)])
+@pytest.mark.parametrize("M", [1, 2, 3, 8, 16])
+def test_edge_shapes(engine, oracle, gpu, N, K, M):
+    run_case(engine, oracle, gpu, N, K, M, engine.META_F16_INTERLEAVED, engine.F16, engine.F32)
+
+
+@pytest.mark.parametrize("name,N,K", [("q", 6144, 5120), ("kv", 1024, 5120), ("o", 5120, 6144),
+                                      ("gate_up", 17408, 5120), ("down", 5120, 17408)])
+@pytest.mark.parametrize("M", [1, 4, 8])
+def test_27b_layer_shapes(engine, oracle, gpu, name, N, K, M):
+    """BASELINE configs 2 and 3: bf16 scale/bias, fp16 activations, fp16 output."""
+    run_case(engine, oracle, gpu, N, K, M, engine.META_BF16_PLANES, engine.F16, engine.F16,
+             seed=11)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_fp32_activations(engine, oracle, gpu, M):
+    """fp32 x (the reference's cpu_q4_dot_float, qwen38_m3_layer.m:375-393) with a residual
+    (qwen38_q4.metal:163-191)."""
+    run_case(engine, oracle, gpu, 5120, 17408 if M == 1 else 2048, M,
+             engine.META_F16_INTERLEAVED, engine.F32, engine.F32, residual=True)
+
+
+@pytest.mark.parametrize("y_dtype", ["F16", "BF16", "F32"])
+def test_bf16_activations_and_outputs(engine, oracle, gpu, y_dtype):
+    """bf16 activations and outputs (minimax_h3_m3_run_q4_projection_bf16)."""
+    run_case(engine, oracle, gpu, 1000, 1536, 5, engine.META_BF16_PLANES, engine.BF16,
+             getattr(engine, y_dtype))
+
+
+def test_repeat_calls_are_bitwise_stable(engine, gpu):
+    """Split-K partial sums are added in a fixed order: same bytes every call."""
+    N, K, M = 5120, 17408, 4
+    quants, meta_a, meta_b = engine.synth_q4_affine(3, 0.02, N, K, engine.META_BF16_PLANES)
+    x = make_x(engine, 5, M, K, engine.F16)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+    try:
+        first = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+        for _ in range(5):
+            again = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+            assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+    finally:
+        weight.destroy()
+
+
+def test_argument_errors(engine, gpu):
+    quants, meta_a, meta_b = engine.synth_q4_affine(1, 0.02, 16, 64, engine.META_F16_INTERLEAVED)
+    with pytest.raises(engine.Mi355qError) as info:
+        gpu.q4_prepare(quants, meta_a, None, 16, 96, engine.META_F16_INTERLEAVED)
+    assert info.value.status == engine.ERROR_INVALID
+    with pytest.raises(engine.Mi355qError) as info:
+        gpu.q4_prepare(quants, meta_a, None, 16, 64, engine.META_BF16_PLANES)
+    assert info.value.status == engine.ERROR_INVALID
+    weight = gpu.q4_prepare(quants, meta_a, None, 16, 64, engine.META_F16_INTERLEAVED)
+    try:
+        with pytest.raises(engine.Mi355qError) as info:
+            gpu.q4_linear(weight, np.zeros((0, 64), np.float16), engine.F16)
+        assert info.value.status == engine.ERROR_INVALID
+    finally:
+        weight.destroy()
