@@ -24,33 +24,6 @@ int fail_hip(hipError_t status, const char *what, char *error, size_t capacity)
     return MI355Q_ERROR_RUNTIME;
 }
 
-int ensure_partials(mi355q_context *ctx, size_t bytes, size_t counters,
-                    char *error, size_t error_capacity)
-{
-    if (bytes > ctx->partials_bytes) {
-        MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before workspace growth");
-        if (ctx->partials) (void)hipFree(ctx->partials);
-        ctx->partials = nullptr;
-        ctx->partials_bytes = 0;
-        size_t want = bytes + bytes / 2;
-        MI355Q_HIP(hipMalloc((void **)&ctx->partials, want), "workspace allocation");
-        ctx->partials_bytes = want;
-    }
-    if (counters > ctx->counters_count) {
-        MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before counter growth");
-        if (ctx->counters) (void)hipFree(ctx->counters);
-        ctx->counters = nullptr;
-        ctx->counters_count = 0;
-        size_t want = counters * 2;
-        MI355Q_HIP(hipMalloc((void **)&ctx->counters, want * sizeof(uint32_t)),
-                   "counter allocation");
-        MI355Q_HIP(hipMemsetAsync(ctx->counters, 0, want * sizeof(uint32_t), ctx->stream),
-                   "counter clear");
-        ctx->counters_count = want;
-    }
-    return MI355Q_OK;
-}
-
 int ensure_stage(mi355q_context *ctx, int slot, size_t bytes, char *error,
                  size_t error_capacity)
 {
@@ -117,9 +90,7 @@ void mi355q_context_destroy(mi355q_context *ctx)
     if (ctx == nullptr) return;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    if (ctx->partials) (void)hipFree(ctx->partials);
-    if (ctx->counters) (void)hipFree(ctx->counters);
-    for (int slot = 0; slot < 3; ++slot)
+    for (int slot = 0; slot < 4; ++slot)
         if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
     if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
     if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
@@ -429,6 +400,27 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const 
                    "output download");
     if (!(flags & MI355Q_ASYNC))
         MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear sync");
+    return MI355Q_OK;
+}
+
+int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,
+                              char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || (calls == nullptr && count != 0)) {
+        set_error(error, error_capacity, "q4_linear_sequence: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    const uint32_t flags = MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE | MI355Q_ASYNC;
+    for (size_t i = 0; i < count; ++i) {
+        const mi355q_q4_call &c = calls[i];
+        char inner[256] = "";
+        int status = mi355q_q4_linear(ctx, c.weight, c.x, c.x_dtype, c.M, c.y, c.y_dtype,
+                                      c.residual, c.residual_dtype, flags, inner, sizeof inner);
+        if (status != MI355Q_OK) {
+            set_error(error, error_capacity, "call %zu: %s", i, inner);
+            return status;
+        }
+    }
     return MI355Q_OK;
 }
 

@@ -18,8 +18,10 @@ namespace mi355q {
 // its 16 bytes at offset 16*l.  Lane l = (row r = l % 16, quarter kq = l / 16)
 // holds four dwords; dword d is the row's original little-endian code word
 // number 4*d + kq of the 16 words in the 128-column step, i.e. columns
-// 32*d + 8*kq .. +7.  One 16x16x32 MFMA therefore consumes dword d of every
-// lane and covers the contiguous columns 32*d .. 32*d+31 (half a group).
+// 32*d + 8*kq .. +7, with its nibbles regrouped (even columns in the low half,
+// odd columns in the high half) so that the two-at-a-time unpack yields column
+// order.  One 16x16x32 MFMA therefore consumes dword d of every lane and
+// covers the contiguous columns 32*d .. 32*d+31 (half a group).
 // Metadata: per (tile, step, row) eight bytes = {scale,bias} of group 2*step
 // then of group 2*step+1, 16-bit fields in the image's own encoding.
 // Rows beyond N and columns beyond K are padded with zero codes and zero
@@ -43,15 +45,9 @@ struct mi355q_context {
     hipEvent_t timer_start, timer_stop;
     bool timer_open;
     hipDeviceProp_t props;
-    // split-K workspace: fp32 partial sums and one arrival counter per
-    // workgroup column; counters are zero between calls.
-    float *partials;
-    size_t partials_bytes;
-    uint32_t *counters;
-    size_t counters_count;
-    // staging for host-pointer activations / outputs
-    void *stage[3];
-    size_t stage_bytes[3];
+    // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16
+    void *stage[4];
+    size_t stage_bytes[4];
 };
 
 struct mi355q_q4_weight {
@@ -72,8 +68,6 @@ int fail_hip(hipError_t status, const char *what, char *error, size_t capacity);
             return ::mi355q::fail_hip(status_, what, error, error_capacity); \
     } while (0)
 
-int ensure_partials(mi355q_context *ctx, size_t bytes, size_t counters,
-                    char *error, size_t error_capacity);
 int ensure_stage(mi355q_context *ctx, int slot, size_t bytes,
                  char *error, size_t error_capacity);
 

@@ -25,9 +25,14 @@ q4_repack_codes_kernel(const uint32_t *__restrict__ src_words, uint4 *__restrict
 #pragma unroll
     for (uint32_t d = 0; d < 4; ++d) {
         uint32_t word = step * 16u + 4u * d + kq;
-        out[d] = (row < N && word < words_per_row)
-                     ? src_words[(uint64_t)row * words_per_row + word]
-                     : 0u;
+        uint32_t v = (row < N && word < words_per_row)
+                         ? src_words[(uint64_t)row * words_per_row + word]
+                         : 0u;
+        // even columns to the low half, odd columns to the high half
+        uint32_t even = (v & 0xFu) | ((v >> 4) & 0xF0u) | ((v >> 8) & 0xF00u) | ((v >> 12) & 0xF000u);
+        uint32_t odd = ((v >> 4) & 0xFu) | ((v >> 8) & 0xF0u) | ((v >> 12) & 0xF00u) |
+                       ((v >> 16) & 0xF000u);
+        out[d] = even | (odd << 16);
     }
     dst[index] = make_uint4(out[0], out[1], out[2], out[3]);
 }

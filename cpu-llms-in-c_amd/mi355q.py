@@ -41,6 +41,11 @@ class DeviceInfo(_c.Structure):
     ]
 
 
+class Q4Call(_c.Structure):
+    _fields_ = [("weight", _vp), ("x", _vp), ("y", _vp), ("residual", _vp), ("M", _u32),
+                ("x_dtype", _int), ("y_dtype", _int), ("residual_dtype", _int)]
+
+
 # name -> (restype, argtypes): every symbol the two headers declare
 SIGNATURES = {
     "mi355q_context_create": (_int, [_int, _c.POINTER(_vp), *_err]),
@@ -53,11 +58,13 @@ SIGNATURES = {
     "mi355q_download": (_int, [_vp, _vp, _vp, _sz, *_err]),
     "mi355q_timer_begin": (_int, [_vp, *_err]),
     "mi355q_timer_end": (_int, [_vp, _c.POINTER(_c.c_double), *_err]),
+    "mi355q_probe_read_bandwidth": (_int, [_vp, _sz, _sz, _int, _int, _c.POINTER(_c.c_double), *_err]),
     "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
                                         _c.POINTER(_vp), *_err]),
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
+    "mi355q_q4_linear_sequence": (_int, [_vp, _c.POINTER(Q4Call), _sz, *_err]),
     "mi355q_synth_normal_f32": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_synth_normal_f16": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_quantize_q4_affine": (_int, [_vp, _u32, _u32, _int, _vp, _vp, _vp]),
@@ -183,6 +190,13 @@ class Context:
         _call(self.lib.mi355q_timer_end, self.handle, ctypes.byref(ms))
         return ms.value
 
+    def probe_read_bandwidth(self, nbytes: int = 2 << 30, repeats: int = 5, variant: int = 1,
+                             launch_bytes: int = 0) -> float:
+        gbs = ctypes.c_double()
+        _call(self.lib.mi355q_probe_read_bandwidth, self.handle, nbytes, launch_bytes, repeats, variant,
+              ctypes.byref(gbs))
+        return gbs.value
+
     # ---- affine Q4 ----
     def q4_prepare(self, quants, meta_a, meta_b, N: int, K: int, meta_kind: int,
                    flags: int = 0) -> Q4Weight:
@@ -207,6 +221,23 @@ class Context:
         flags = X_DEVICE | Y_DEVICE | RESIDUAL_DEVICE | (ASYNC if asynchronous else 0)
         _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, x_ptr, x_dtype, M, y_ptr,
               y_dtype, residual_ptr, residual_dtype, flags)
+
+    def q4_sequence(self, calls):
+        """calls: a ctypes array of Q4Call (build once, reuse)."""
+        _call(self.lib.mi355q_q4_linear_sequence, self.handle, calls, len(calls))
+
+
+def make_calls(items):
+    """items: iterable of (weight, x_ptr, x_dtype, M, y_ptr, y_dtype[, residual_ptr, residual_dtype])."""
+    items = list(items)
+    array = (Q4Call * len(items))()
+    for slot, item in zip(array, items):
+        weight, x_ptr, x_dtype, M, y_ptr, y_dtype = item[:6]
+        slot.weight, slot.x, slot.y = weight.handle, x_ptr, y_ptr
+        slot.M, slot.x_dtype, slot.y_dtype = M, x_dtype, y_dtype
+        slot.residual = item[6] if len(item) > 6 else None
+        slot.residual_dtype = item[7] if len(item) > 7 else F32
+    return array
 
 
 # ---- synthetic inputs (host side) ------------------------------------------

@@ -110,6 +110,18 @@ int mi355q_timer_begin(mi355q_context *ctx, char *error, size_t error_capacity);
 int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms,
                      char *error, size_t error_capacity);
 
+/* Measured read bandwidth of HBM: one pass of 128-bit loads over a private
+ * buffer of `bytes` (use >= 1 GiB to defeat the 256 MB memory-side cache),
+ * best of `repeats`.  `launch_bytes` (0 = the whole buffer) splits the pass
+ * into back-to-back kernel launches of that size each, which shows what a
+ * kernel as short as one weight matrix can reach.  variant 0: plain loads,
+ * 1: streaming (non-temporal) loads, 2: plain loads with a larger grid.  The
+ * analogue of the reference's bandwidth probes (tools/target_probe.c;
+ * qwen38_jetson_memory_probe.cu:25-35). */
+int mi355q_probe_read_bandwidth(mi355q_context *ctx, size_t bytes, size_t launch_bytes,
+                                int repeats, int variant, double *gb_per_s,
+                                char *error, size_t error_capacity);
+
 /* ---- affine Q4, group 64: w[n][k] = scale[n][k/64] * q[n][k] + bias[n][k/64]
  *
  * quants: [N][K/64][32] bytes, element k of a row in byte k/2, even k in the
@@ -145,6 +157,23 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight,
                      void *y, int y_dtype,
                      const void *residual, int residual_dtype,
                      uint32_t flags, char *error, size_t error_capacity);
+
+/* A run of linears queued back to back on the context's stream with one host
+ * call, all pointers on the device and nothing waited for — the way the
+ * reference encodes every matvec of a forward pass into one command buffer
+ * before committing it (qwen38_m3_decode.m:1614-1699).  Stops at the first
+ * call that fails and reports its index in the message. */
+typedef struct {
+    const mi355q_q4_weight *weight;
+    const void *x;
+    void *y;
+    const void *residual; /* or NULL */
+    uint32_t M;
+    int x_dtype, y_dtype, residual_dtype;
+} mi355q_q4_call;
+
+int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,
+                              size_t count, char *error, size_t error_capacity);
 
 #ifdef __cplusplus
 }
