@@ -66,7 +66,9 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     }
     memset(ctx, 0, sizeof *ctx);
     ctx->device = device;
-    hipError_t status = hipGetDeviceProperties(&ctx->props, device);
+    ctx->profile_events = new (std::nothrow) std::vector<hipEvent_t>();
+    hipError_t status = ctx->profile_events ? hipSuccess : hipErrorOutOfMemory;
+    if (status == hipSuccess) status = hipGetDeviceProperties(&ctx->props, device);
     if (status == hipSuccess && strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
         set_error(error, error_capacity, "context_create: device is %s, kernels are built for gfx950",
                   ctx->props.gcnArchName);
@@ -92,6 +94,10 @@ void mi355q_context_destroy(mi355q_context *ctx)
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (int slot = 0; slot < 4; ++slot)
         if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
+    if (ctx->profile_events) {
+        for (hipEvent_t event : *ctx->profile_events) (void)hipEventDestroy(event);
+        delete ctx->profile_events;
+    }
     if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
     if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -207,6 +213,39 @@ int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms, char *error,
     MI355Q_HIP(hipEventElapsedTime(&ms, ctx->timer_start, ctx->timer_stop),
                "hipEventElapsedTime");
     *gpu_ms = (double)ms;
+    return MI355Q_OK;
+}
+
+int mi355q_profile_begin(mi355q_context *ctx, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr) {
+        set_error(error, error_capacity, "profile_begin: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    ctx->profiling = true;
+    ctx->profile_used = 0;
+    return MI355Q_OK;
+}
+
+int mi355q_profile_end(mi355q_context *ctx, double *kernel_ms, uint64_t *launches, char *error,
+                       size_t error_capacity)
+{
+    if (ctx == nullptr || kernel_ms == nullptr || !ctx->profiling) {
+        set_error(error, error_capacity, "profile_end: no profile_begin on this context");
+        return MI355Q_ERROR_INVALID;
+    }
+    ctx->profiling = false;
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    double total = 0.0;
+    for (size_t i = 0; i + 1 < ctx->profile_used; i += 2) {
+        float ms = 0.0f;
+        MI355Q_HIP(hipEventElapsedTime(&ms, (*ctx->profile_events)[i], (*ctx->profile_events)[i + 1]),
+                   "hipEventElapsedTime");
+        total += (double)ms;
+    }
+    *kernel_ms = total;
+    if (launches) *launches = ctx->profile_used / 2;
     return MI355Q_OK;
 }
 

@@ -2,11 +2,13 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <vector>
 
 #include "mi355q.h"
 
@@ -24,14 +26,18 @@ namespace mi355q {
 // covers the contiguous columns 32*d .. 32*d+31 (half a group).
 // Metadata: per (tile, step, row) eight bytes = {scale,bias} of group 2*step
 // then of group 2*step+1, 16-bit fields in the image's own encoding.
-// Rows beyond N and columns beyond K are padded with zero codes and zero
-// metadata, which contribute exactly 0.
+// Records are stored step-major, record(step, tile) = step * NT + tile: the
+// waves of all workgroups advance through the steps at about the same pace, so
+// at any moment the chip reads a few compact regions of HBM (one per step in
+// flight) instead of one scattered kilobyte per tile, which keeps DRAM pages
+// open.  Rows beyond N and columns beyond K are padded with zero codes and
+// zero metadata, which contribute exactly 0.
 constexpr uint32_t kTileRows = 16;
 constexpr uint32_t kStepColumns = 128;
 
 struct Q4Device {
-    uint4 *codes;   // [NT][T][64]
-    uint2 *meta;    // [NT][T][16]
+    uint4 *codes;   // [T][NT][64]
+    uint2 *meta;    // [T][NT][16]
     uint32_t N, K;  // logical shape
     uint32_t NT, T; // tiles of 16 rows, steps of 128 columns
     int meta_kind;
@@ -45,6 +51,11 @@ struct mi355q_context {
     hipEvent_t timer_start, timer_stop;
     bool timer_open;
     hipDeviceProp_t props;
+    // per-kernel timing between profile_begin and profile_end: one event pair
+    // per launch, bound to the dispatch's own start and end
+    bool profiling;
+    std::vector<hipEvent_t> *profile_events;
+    size_t profile_used;
     // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16
     void *stage[4];
     size_t stage_bytes[4];
@@ -70,6 +81,29 @@ int fail_hip(hipError_t status, const char *what, char *error, size_t capacity);
 
 int ensure_stage(mi355q_context *ctx, int slot, size_t bytes,
                  char *error, size_t error_capacity);
+
+// Every compute kernel goes through here so that profiling sees it.
+template <typename Kernel, typename... Args>
+hipError_t launch(mi355q_context *ctx, Kernel kernel, dim3 grid, dim3 block, size_t lds,
+                  Args... args)
+{
+    if (ctx->profiling) {
+        std::vector<hipEvent_t> &events = *ctx->profile_events;
+        while (events.size() < ctx->profile_used + 2) {
+            hipEvent_t fresh;
+            hipError_t created = hipEventCreate(&fresh);
+            if (created != hipSuccess) return created;
+            events.push_back(fresh);
+        }
+        hipEvent_t start = events[ctx->profile_used], stop = events[ctx->profile_used + 1];
+        ctx->profile_used += 2;
+        hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds, ctx->stream, start, stop, 0,
+                              args...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, args...);
+    }
+    return hipGetLastError();
+}
 
 inline size_t dtype_bytes(int dtype) { return dtype == MI355Q_F32 ? 4u : 2u; }
 inline bool dtype_valid(int dtype) {

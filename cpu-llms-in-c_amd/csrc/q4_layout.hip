@@ -15,9 +15,9 @@ q4_repack_codes_kernel(const uint32_t *__restrict__ src_words, uint4 *__restrict
     uint64_t total = (uint64_t)NT * T * 64u;
     if (index >= total) return;
     uint32_t lane = (uint32_t)(index & 63u);
-    uint64_t tile_step = index >> 6;
-    uint32_t step = (uint32_t)(tile_step % T);
-    uint32_t tile = (uint32_t)(tile_step / T);
+    uint64_t record = index >> 6;  // step-major: record = step * NT + tile
+    uint32_t tile = (uint32_t)(record % NT);
+    uint32_t step = (uint32_t)(record / NT);
     uint32_t row = tile * kTileRows + (lane & 15u);
     uint32_t kq = lane >> 4;
     uint32_t words_per_row = K / 8u;
@@ -49,9 +49,9 @@ q4_repack_meta_kernel(const uint16_t *__restrict__ meta_a,
     uint64_t total = (uint64_t)NT * T * 16u;
     if (index >= total) return;
     uint32_t r = (uint32_t)(index & 15u);
-    uint64_t tile_step = index >> 4;
-    uint32_t step = (uint32_t)(tile_step % T);
-    uint32_t tile = (uint32_t)(tile_step / T);
+    uint64_t record = index >> 4;  // step-major: record = step * NT + tile
+    uint32_t tile = (uint32_t)(record % NT);
+    uint32_t step = (uint32_t)(record / NT);
     uint32_t row = tile * kTileRows + r;
     uint32_t groups = K / 64u;
     uint32_t out[2];

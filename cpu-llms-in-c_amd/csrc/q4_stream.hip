@@ -12,8 +12,7 @@
 //
 // Work split: a workgroup owns TB tiles (16 output rows each) and keeps the
 // activations in LDS.  Its W waves take the 128-column steps round-robin (wave
-// w: steps w, w+W, ...), so the workgroup reads W KiB of contiguous codes per
-// tile at a time; each wave keeps D steps of loads in flight.  Partial sums
+// w: steps w, w+W, ...); each wave keeps D steps of loads in flight.  Partial sums
 // meet in LDS and are added in wave order (a fixed order: results do not
 // depend on timing).  Nothing is shared between workgroups.  Long rows with
 // many activation rows are walked in column chunks so the activations fit LDS.
@@ -69,8 +68,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     for (int tb = 0; tb < TB; ++tb) {
         uint32_t tile = tile0 + tb;
         tile = tile < p.NT ? tile : p.NT - 1u;
-        codes_tile[tb] = p.codes + (size_t)tile * p.T * 64u + lane;
-        meta_tile[tb] = p.meta + (size_t)tile * p.T * 16u + r;
+        codes_tile[tb] = p.codes + (size_t)tile * 64u + lane;
+        meta_tile[tb] = p.meta + (size_t)tile * 16u + r;
     }
 
     floatx4 acc[TB];
@@ -98,25 +97,44 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             step = step < p.T ? step : p.T - 1u;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * 16u);
+                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * p.NT * 64u);
+                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * p.NT * 16u);
             }
         };
+        // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
+        // The activation loads go out first (they come back from L2 quickly),
+        // then the first D weight steps; the LDS stores wait for the former only.
+        constexpr int SB = 4;
+        const uint32_t octets = span * 16u;
+        const uint32_t items = octets * MP;
+        auto stage_fetch = [&](uint32_t index) {
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (index < items) {
+                const uint32_t mrow = index / octets, o = index % octets;
+                const uint32_t k = first * kStepColumns + o * 8u;
+                if (mrow < p.rows && k < p.K) v = *(const uint4 *)(p.x + (size_t)mrow * p.K + k);
+            }
+            return v;
+        };
+        auto stage_store = [&](uint32_t index, const uint4 &v) {
+            if (index < items) xs[(size_t)(index % octets) * MP + index / octets] = v;
+        };
+        uint4 staged[SB];
+#pragma unroll
+        for (int b = 0; b < SB; ++b) staged[b] = stage_fetch(threadIdx.x + b * 64u * W);
+
         StepData<TB> ring[D];
 #pragma unroll
         for (int u = 0; u < D; ++u) issue(u, ring[u]);
 
-        // ---- activations of this chunk into LDS: [octet][row], 16 bytes each
         if (chunk > 0) __syncthreads();  // everyone is done with the previous chunk
-        {
-            const uint32_t octets = span * 16u;
-            for (uint32_t index = threadIdx.x; index < octets * MP; index += 64u * W) {
-                const uint32_t mrow = index / octets, o = index % octets;
-                const uint32_t k = first * kStepColumns + o * 8u;
-                uint4 v = make_uint4(0u, 0u, 0u, 0u);
-                if (mrow < p.rows && k < p.K) v = *(const uint4 *)(p.x + (size_t)mrow * p.K + k);
-                xs[(size_t)o * MP + mrow] = v;
-            }
+#pragma unroll
+        for (int b = 0; b < SB; ++b) stage_store(threadIdx.x + b * 64u * W, staged[b]);
+        for (uint32_t base = threadIdx.x + SB * 64u * W; base < items; base += SB * 64u * W) {
+#pragma unroll
+            for (int b = 0; b < SB; ++b) staged[b] = stage_fetch(base + b * 64u * W);
+#pragma unroll
+            for (int b = 0; b < SB; ++b) stage_store(base + b * 64u * W, staged[b]);
         }
         __syncthreads();
 
@@ -231,31 +249,28 @@ struct StreamShape {
 };
 
 template <int MP, int TB, int D, int W>
-static hipError_t launch_one(const StreamParams &p, hipStream_t stream)
+static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
 {
     constexpr int NJ = MP < 4 ? MP : 4;
     const uint32_t blocks = (p.NT + TB - 1) / TB;
     const size_t lds = (size_t)p.chunk_steps * 16u * MP * sizeof(uint4) +
                        (size_t)W * TB * NJ * 64u * sizeof(float);
     if (p.meta_bf16)
-        hipLaunchKernelGGL((q4_stream_kernel<MP, TB, D, W, true>), dim3(blocks), dim3(64u * W), lds,
-                           stream, p);
-    else
-        hipLaunchKernelGGL((q4_stream_kernel<MP, TB, D, W, false>), dim3(blocks), dim3(64u * W), lds,
-                           stream, p);
-    return hipGetLastError();
+        return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, dim3(blocks), dim3(64u * W), lds, p);
+    return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, dim3(blocks), dim3(64u * W), lds, p);
 }
 
 template <int MP>
-static hipError_t launch_mp(const StreamParams &p, const StreamShape &shape, hipStream_t stream)
+static hipError_t launch_mp(mi355q_context *ctx, const StreamParams &p, const StreamShape &shape)
 {
-    switch (shape.tb * 1000 + shape.depth * 10 + shape.waves) {
-    case 1024: return launch_one<MP, 1, 2, 4>(p, stream);
-    case 1044: return launch_one<MP, 1, 4, 4>(p, stream);
-    case 1028: return launch_one<MP, 1, 2, 8>(p, stream);
-    case 1048: return launch_one<MP, 1, 4, 8>(p, stream);
-    case 2024: return launch_one<MP, 2, 2, 4>(p, stream);
-    case 2028: return launch_one<MP, 2, 2, 8>(p, stream);
+    switch (shape.tb * 10000 + shape.depth * 100 + shape.waves) {
+    case 10202: return launch_one<MP, 1, 2, 2>(ctx, p);
+    case 10204: return launch_one<MP, 1, 2, 4>(ctx, p);
+    case 10208: return launch_one<MP, 1, 2, 8>(ctx, p);
+    case 10404: return launch_one<MP, 1, 4, 4>(ctx, p);
+    case 10408: return launch_one<MP, 1, 4, 8>(ctx, p);
+    case 20204: return launch_one<MP, 2, 2, 4>(ctx, p);
+    case 20208: return launch_one<MP, 2, 2, 8>(ctx, p);
     default: return hipErrorInvalidValue;
     }
 }
@@ -289,9 +304,13 @@ static StreamShape choose_shape(const mi355q_context *ctx, const Q4Device &w, in
     StreamShape shape;
     shape.mp = mp;
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
-    shape.tb = w.NT >= 4u * cus ? 2 : 1;
+    // about 4-5 thousand waves with two steps of loads in flight each keeps HBM
+    // busy without queueing; more waves per workgroup when there are few tiles
+    shape.tb = 1;
     shape.depth = 2;
-    shape.waves = w.T >= 32u ? 8 : 4;
+    const uint32_t want = (16u * cus + w.NT - 1) / w.NT;
+    shape.waves = want <= 2u ? 2 : want <= 5u ? 4 : 8;
+    while (shape.waves > 2 && (uint32_t)shape.waves > w.T) shape.waves /= 2;
     const char *force = getenv("MI355Q_Q4_STREAM");  // "TB,DEPTH,WAVES" for experiments
     int ft = 0, fd = 0, fw = 0;
     if (force && sscanf(force, "%d,%d,%d", &ft, &fd, &fw) == 3) {
@@ -334,9 +353,9 @@ int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs 
         int status = ensure_stage(ctx, 3, bytes, error, error_capacity);
         if (status != MI355Q_OK) return status;
         const size_t count = (size_t)a.M * w.K;
-        hipLaunchKernelGGL(q4_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256),
-                           0, ctx->stream, a.x, a.x_dtype, (_Float16 *)ctx->stage[3], a.M, w.K);
-        hipError_t converted = hipGetLastError();
+        hipError_t converted =
+            launch(ctx, q4_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256), 0,
+                   a.x, a.x_dtype, (_Float16 *)ctx->stage[3], a.M, w.K);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = (const _Float16 *)ctx->stage[3];
@@ -365,11 +384,11 @@ int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs 
     }
     hipError_t launched;
     switch (mp) {
-    case 1: launched = launch_mp<1>(p, shape, ctx->stream); break;
-    case 2: launched = launch_mp<2>(p, shape, ctx->stream); break;
-    case 4: launched = launch_mp<4>(p, shape, ctx->stream); break;
-    case 8: launched = launch_mp<8>(p, shape, ctx->stream); break;
-    default: launched = launch_mp<16>(p, shape, ctx->stream); break;
+    case 1: launched = launch_mp<1>(ctx, p, shape); break;
+    case 2: launched = launch_mp<2>(ctx, p, shape); break;
+    case 4: launched = launch_mp<4>(ctx, p, shape); break;
+    case 8: launched = launch_mp<8>(ctx, p, shape); break;
+    default: launched = launch_mp<16>(ctx, p, shape); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 stream kernel launch", error, error_capacity);

@@ -58,6 +58,8 @@ SIGNATURES = {
     "mi355q_download": (_int, [_vp, _vp, _vp, _sz, *_err]),
     "mi355q_timer_begin": (_int, [_vp, *_err]),
     "mi355q_timer_end": (_int, [_vp, _c.POINTER(_c.c_double), *_err]),
+    "mi355q_profile_begin": (_int, [_vp, *_err]),
+    "mi355q_profile_end": (_int, [_vp, _c.POINTER(_c.c_double), _c.POINTER(_u64), *_err]),
     "mi355q_probe_read_bandwidth": (_int, [_vp, _sz, _sz, _int, _int, _c.POINTER(_c.c_double), *_err]),
     "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
                                         _c.POINTER(_vp), *_err]),
@@ -189,6 +191,15 @@ class Context:
         ms = ctypes.c_double()
         _call(self.lib.mi355q_timer_end, self.handle, ctypes.byref(ms))
         return ms.value
+
+    def profile_begin(self):
+        _call(self.lib.mi355q_profile_begin, self.handle)
+
+    def profile_end(self):
+        """(sum of kernel durations in ms, number of kernel launches)"""
+        ms, launches = ctypes.c_double(), ctypes.c_uint64()
+        _call(self.lib.mi355q_profile_end, self.handle, ctypes.byref(ms), ctypes.byref(launches))
+        return ms.value, launches.value
 
     def probe_read_bandwidth(self, nbytes: int = 2 << 30, repeats: int = 5, variant: int = 1,
                              launch_bytes: int = 0) -> float:

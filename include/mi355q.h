@@ -110,6 +110,15 @@ int mi355q_timer_begin(mi355q_context *ctx, char *error, size_t error_capacity);
 int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms,
                      char *error, size_t error_capacity);
 
+/* Per-kernel GPU time: between the two calls every compute kernel the context
+ * launches carries its own start/stop event pair; `kernel_ms` is the sum of
+ * the kernels' own durations (no gaps between launches) and `launches` their
+ * number.  The reference's QWEN38_PROFILE mode sums GPUEndTime-GPUStartTime per
+ * kernel class the same way (qwen38_m3_decode.m:1217-1283). */
+int mi355q_profile_begin(mi355q_context *ctx, char *error, size_t error_capacity);
+int mi355q_profile_end(mi355q_context *ctx, double *kernel_ms, uint64_t *launches,
+                       char *error, size_t error_capacity);
+
 /* Measured read bandwidth of HBM: one pass of 128-bit loads over a private
  * buffer of `bytes` (use >= 1 GiB to defeat the 256 MB memory-side cache),
  * best of `repeats`.  `launch_bytes` (0 = the whole buffer) splits the pass
