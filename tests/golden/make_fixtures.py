@@ -1,0 +1,78 @@
+"""Writes the golden vectors under tests/golden/ from the reference's own compiled C
+(oracle/_ref, built by oracle/Makefile from the sources under the reference tree).
+Run in the build container only; the committed .npz files are what the tests read
+where the reference tree is absent.  Inputs are seeded; nothing here imports or
+executes the reference's Python.
+
+    python tests/golden/make_fixtures.py
+"""
+import sys
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parents[2]
+sys.path.insert(0, str(ROOT / "oracle"))
+sys.path.insert(0, str(ROOT / "tests"))
+import oracle  # noqa: E402
+from sym128 import output_block, pack_sym128  # noqa: E402
+
+HERE = Path(__file__).resolve().parent
+
+
+def sym128_fixture():
+    ref = oracle.ref_qwen35()
+    assert ref is not None, "oracle/_ref is not built"
+    rng = np.random.default_rng(20250101)
+    rows, cols = 12, 384
+    weights = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    weights[3, 128:256] = 0.0  # an all-zero group (scale falls back to 1)
+    records = pack_sym128(weights)
+    blocked = output_block(records, 4)
+    x = rng.standard_normal(cols).astype(np.float32)
+    out = {"weights": weights, "records": records.reshape(-1), "blocked": blocked, "x": x}
+    for name, data, flag in (("rowmajor", records.reshape(-1), 0), ("blocked", blocked, 1)):
+        y = np.empty(rows, dtype=np.float32)
+        ref.ref_qwen35_q4_gemv(data.ctypes.data, flag, rows, cols, x.ctypes.data, y.ctypes.data)
+        out[f"y_{name}"] = y
+        dq = np.empty((rows, cols), dtype=np.float32)
+        for r in range(rows):
+            ref.ref_qwen35_dequantize_q4_row(data.ctypes.data, flag, rows, cols, r, dq[r].ctypes.data)
+        out[f"dequant_{name}"] = dq
+    np.savez_compressed(HERE / "sym128_q4_gemv.npz", **out)
+
+
+def w8a8_fixture():
+    ref = oracle.ref_minimindo()
+    assert ref is not None, "oracle/_ref is not built"
+    rng = np.random.default_rng(20250102)
+    M, K, N = 7, 160, 24
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    x[2] = 0.0                      # all-zero token: zero codes, scale 0
+    x[3, :8] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.0, -127.0]  # exact .5 ties after scaling
+    x[3, 8:] = 0.0
+    x[3, 6] = 127.0
+    q = np.empty((M, K), dtype=np.int8)
+    scales = np.empty(M, dtype=np.float32)
+    for m in range(M):
+        scales[m] = ref.ref_minimindo_quantize_i8(x[m].ctypes.data, q[m].ctypes.data, K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    rows = oracle.q8_weight_quantize(w)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out_bias = np.empty((M, N), dtype=np.float32)
+    out_nobias = np.empty((M, N), dtype=np.float32)
+    ref.ref_minimindo_matrix_sequence_i8_quantized(rows.ctypes.data, N, K, q.ctypes.data,
+                                                   scales.ctypes.data, M, out_bias.ctypes.data,
+                                                   bias.ctypes.data)
+    ref.ref_minimindo_matrix_sequence_i8_quantized(rows.ctypes.data, N, K, q.ctypes.data,
+                                                   scales.ctypes.data, M, out_nobias.ctypes.data, None)
+    dots = np.array([[ref.ref_minimindo_q8_i8_dot(rows[n * (4 + K) + 4:].ctypes.data, q[m].ctypes.data, K)
+                      for n in range(N)] for m in range(M)], dtype=np.int32)
+    np.savez_compressed(HERE / "w8a8_minimindo.npz", x=x, q=q, scales=scales, w=w, rows=rows, bias=bias,
+                        out_bias=out_bias, out_nobias=out_nobias, dots=dots)
+
+
+if __name__ == "__main__":
+    sym128_fixture()
+    w8a8_fixture()
+    print("wrote", sorted(p.name for p in HERE.glob("*.npz")))
