@@ -92,7 +92,7 @@ void mi355q_context_destroy(mi355q_context *ctx)
     if (ctx == nullptr) return;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    for (int slot = 0; slot < 4; ++slot)
+    for (int slot = 0; slot < 5; ++slot)
         if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
     if (ctx->profile_events) {
         for (hipEvent_t event : *ctx->profile_events) (void)hipEventDestroy(event);
@@ -429,8 +429,7 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const 
     if (stream_rows <= 16u) {
         status = q4_stream_linear(ctx, dev, args, error, error_capacity);
     } else {
-        set_error(error, error_capacity, "q4_linear: M=%u is not supported yet", M);
-        status = MI355Q_ERROR_INVALID;
+        status = q4_gemm_linear(ctx, dev, args, error, error_capacity);
     }
     if (status != MI355Q_OK) return status;
 

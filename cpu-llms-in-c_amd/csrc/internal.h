@@ -56,9 +56,10 @@ struct mi355q_context {
     bool profiling;
     std::vector<hipEvent_t> *profile_events;
     size_t profile_used;
-    // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16
-    void *stage[4];
-    size_t stage_bytes[4];
+    // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16,
+    // 4 fp32 partial sums of a K-split GEMM
+    void *stage[5];
+    size_t stage_bytes[5];
 };
 
 struct mi355q_q4_weight {
@@ -127,5 +128,8 @@ struct Q4LinearArgs {
 };
 int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
                      char *error, size_t error_capacity);
+// q4_gemm.hip
+int q4_gemm_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
+                   char *error, size_t error_capacity);
 
 }  // namespace mi355q

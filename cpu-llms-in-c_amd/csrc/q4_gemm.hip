@@ -1,0 +1,273 @@
+// Prefill GEMM on affine-Q4 weights: y[M][N] = x[M][K] * w[N][K]^T for M > 16.
+// MFMA-bound.  The reference's batched kernels dequantize a weight tile to half
+// precision and multiply it with 8x8 simdgroup MMAs, accumulating in fp32
+// (qwen38_prefill.metal:953-1078,1373-1502; minimax_h3_attention.metal:211-592);
+// its scalar check rounds the weight to fp16 the same way
+// (minimax_h3_m3_gemm.m:87-104).  Here: w16 = fp16(s*q + b) (one fused fp16
+// multiply-add per weight), fp16 x fp16 products on v_mfma_f32_16x16x32_f16,
+// fp32 accumulation over the whole of K.
+//
+// Work split: a workgroup of four waves computes a 128 (rows of x) by 64*NTW
+// (rows of w) block of y.  The activations of one 128-column step are staged in
+// LDS (double buffered) and shared by the four waves; every wave dequantizes
+// the codes of its own NTW tiles of 16 weight rows straight into the B-operand
+// registers of the matrix instruction (the stream-tile layout hands each lane
+// exactly the eight consecutive columns the instruction wants), so each weight
+// is dequantized once per workgroup and never passes through LDS.
+#include "device_util.h"
+#include "internal.h"
+
+#include <cstring>
+
+namespace mi355q {
+
+constexpr int kGemmBM = 128;  // rows of x per workgroup
+
+struct GemmParams {
+    const uint4 *codes;
+    const uint2 *meta;
+    const _Float16 *x;  // [M][K] fp16
+    void *y;
+    const void *residual;
+    float *partials;    // [splits][M][N] when splits > 1
+    uint32_t M, N, K, NT, T;
+    uint32_t splits, steps_per_split;
+    int y_dtype, residual_dtype;
+};
+
+__device__ __forceinline__ half8 dequant8(uint32_t word, const NibbleMasks &masks, half8 scale,
+                                          half8 bias)
+{
+    return __builtin_elementwise_fma(unpack8(word, masks), scale, bias);
+}
+
+template <bool BF>
+__device__ __forceinline__ void meta_to_half(uint32_t word, half8 &scale, half8 &bias)
+{
+    _Float16 s, b;
+    if (BF) {
+        s = (_Float16)__builtin_bit_cast(float, word << 16);
+        b = (_Float16)__builtin_bit_cast(float, word & 0xffff0000u);
+    } else {
+        s = __builtin_bit_cast(_Float16, (uint16_t)(word & 0xffffu));
+        b = __builtin_bit_cast(_Float16, (uint16_t)(word >> 16));
+    }
+    scale = half8{s, s, s, s, s, s, s, s};
+    bias = half8{b, b, b, b, b, b, b, b};
+}
+
+template <int NTW, bool BF>
+__global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
+{
+    // activation stage: [buffer][column octet][row ^ octet] of 16-byte pieces; the
+    // XOR spreads the 16 octets a quarter-wave writes for one row over the banks
+    // and keeps the 16 rows a quarter-wave reads for one octet contiguous
+    __shared__ uint4 a_lds[2][16][kGemmBM];
+    constexpr int MI = kGemmBM / 16;  // 16-row fragments of x per workgroup
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15u;
+    const uint32_t kq = lane >> 4;
+    const uint32_t m0 = blockIdx.y * kGemmBM;
+    const uint32_t tile0 = (blockIdx.x * 4u + wave) * NTW;
+    const uint32_t split = blockIdx.z;
+    const uint32_t step_begin = split * p.steps_per_split;
+    const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
+
+    // this thread's part of the activation stage: rows (t/16 + 16*i), octet t%16
+    const uint32_t a_row = threadIdx.x >> 4, a_oct = threadIdx.x & 15u;
+    auto fetch_a = [&](uint32_t step, uint4 (&regs)[MI]) {
+        const uint32_t k = step * kStepColumns + a_oct * 8u;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const uint32_t m = m0 + a_row + 16u * i;
+            regs[i] = (m < p.M && k < p.K) ? *(const uint4 *)(p.x + (size_t)m * p.K + k)
+                                           : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    auto store_a = [&](int buffer, const uint4 (&regs)[MI]) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) a_lds[buffer][a_oct][(a_row + 16u * i) ^ a_oct] = regs[i];
+    };
+    uint4 b_codes[NTW];
+    uint2 b_meta[NTW];
+    auto fetch_b = [&](uint32_t step, uint4 (&codes)[NTW], uint2 (&meta)[NTW]) {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) {
+            uint32_t tile = tile0 + t;
+            tile = tile < p.NT ? tile : p.NT - 1u;  // stay in bounds; such columns are never stored
+            const size_t record = (size_t)step * p.NT + tile;
+            codes[t] = p.codes[record * 64u + lane];
+            meta[t] = p.meta[record * 16u + r];
+        }
+    };
+
+    floatx4 acc[MI][NTW];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) acc[i][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    const NibbleMasks masks = nibble_masks();
+
+    uint4 a_regs[MI];
+    if (step_begin < step_end) {
+        fetch_a(step_begin, a_regs);
+        fetch_b(step_begin, b_codes, b_meta);
+        store_a(0, a_regs);
+    }
+    for (uint32_t step = step_begin; step < step_end; ++step) {
+        const int buffer = (int)((step - step_begin) & 1u);
+        const bool more = step + 1u < step_end;
+        uint4 next_codes[NTW];
+        uint2 next_meta[NTW];
+        if (more) {
+            fetch_a(step + 1u, a_regs);
+            fetch_b(step + 1u, next_codes, next_meta);
+        }
+        __syncthreads();  // stage `buffer` is complete; the other one is free again
+
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            half8 b_frag[NTW];
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) {
+                half8 scale, bias;
+                meta_to_half<BF>(d < 2 ? b_meta[t].x : b_meta[t].y, scale, bias);
+                const uint32_t word = d == 0 ? b_codes[t].x : d == 1 ? b_codes[t].y
+                                      : d == 2 ? b_codes[t].z : b_codes[t].w;
+                b_frag[t] = dequant8(word, masks, scale, bias);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const half8 a_frag = __builtin_bit_cast(half8, a_lds[buffer][4 * d + kq][(16 * i + r) ^ (4 * d + kq)]);
+#pragma unroll
+                for (int t = 0; t < NTW; ++t)
+                    acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag, b_frag[t], acc[i][t],
+                                                                       0, 0, 0);
+            }
+        }
+        if (more) {
+            store_a(buffer ^ 1, a_regs);
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) {
+                b_codes[t] = next_codes[t];
+                b_meta[t] = next_meta[t];
+            }
+        }
+    }
+
+    // ---- lane (r, kq) holds rows 16*i + 4*kq + j of column tile*16 + r
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        const uint32_t tile = tile0 + t;
+        const uint32_t n = tile * kTileRows + r;
+        if (tile >= p.NT || n >= p.N) continue;
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t m = m0 + 16u * i + 4u * kq + j;
+                if (m >= p.M) continue;
+                const size_t at = (size_t)m * p.N + n;
+                if (p.splits > 1u) {
+                    p.partials[(size_t)split * p.M * p.N + at] = acc[i][t][j];
+                } else {
+                    float value = acc[i][t][j];
+                    if (p.residual) value += load_as_float(p.residual, p.residual_dtype, at);
+                    store_from_float(p.y, p.y_dtype, at, value);
+                }
+            }
+    }
+}
+
+// Adds the K splits in split order (a fixed order) and applies the epilogue.
+__global__ void __launch_bounds__(256) q4_gemm_reduce_kernel(const GemmParams p)
+{
+    const size_t total = (size_t)p.M * p.N;
+    const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= total) return;
+    float value = 0.0f;
+    for (uint32_t s = 0; s < p.splits; ++s) value += p.partials[(size_t)s * total + at];
+    if (p.residual) value += load_as_float(p.residual, p.residual_dtype, at);
+    store_from_float(p.y, p.y_dtype, at, value);
+}
+
+// fp32 / bf16 activations are rounded to fp16 once per call (the matrix
+// instruction multiplies fp16 operands).
+__global__ void __launch_bounds__(256)
+q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__restrict__ out,
+                         size_t count)
+{
+    const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= count) return;
+    out[index] = (_Float16)load_as_float(x, x_dtype, index);
+}
+
+int q4_gemm_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a, char *error,
+                   size_t error_capacity)
+{
+    GemmParams p;
+    memset(&p, 0, sizeof p);
+    p.codes = w.codes;
+    p.meta = w.meta;
+    p.x = (const _Float16 *)a.x;
+    if (a.x_dtype != MI355Q_F16) {
+        const size_t count = (size_t)a.M * w.K;
+        int status = ensure_stage(ctx, 3, count * sizeof(_Float16), error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        hipError_t converted =
+            launch(ctx, q4_gemm_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256),
+                   0, a.x, a.x_dtype, (_Float16 *)ctx->stage[3], count);
+        if (converted != hipSuccess)
+            return fail_hip(converted, "activation conversion launch", error, error_capacity);
+        p.x = (const _Float16 *)ctx->stage[3];
+    }
+    p.y = a.y;
+    p.residual = a.residual;
+    p.M = a.M;
+    p.N = w.N;
+    p.K = w.K;
+    p.NT = w.NT;
+    p.T = w.T;
+    p.y_dtype = a.y_dtype;
+    p.residual_dtype = a.residual_dtype;
+
+    constexpr int NTW = 4;
+    const uint32_t n_blocks = (w.NT + 4u * NTW - 1) / (4u * NTW);
+    const uint32_t m_blocks = (a.M + kGemmBM - 1) / kGemmBM;
+    // split K when the output alone does not give every compute unit a block
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    uint32_t splits = 1;
+    const uint32_t blocks = n_blocks * m_blocks;
+    if (blocks < cus) {
+        splits = cus / blocks;
+        if (splits > w.T / 8u) splits = w.T / 8u;
+        if (splits < 1u) splits = 1u;
+    }
+    p.steps_per_split = (w.T + splits - 1) / splits;
+    p.splits = (w.T + p.steps_per_split - 1) / p.steps_per_split;
+    if (p.splits > 1u) {
+        const size_t bytes = (size_t)p.splits * a.M * w.N * sizeof(float);
+        int status = ensure_stage(ctx, 4, bytes, error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        p.partials = (float *)ctx->stage[4];
+    }
+    const dim3 grid(n_blocks, m_blocks, p.splits);
+    hipError_t launched =
+        w.meta_kind == MI355Q_META_BF16_PLANES
+            ? launch(ctx, q4_gemm_kernel<NTW, true>, grid, dim3(256), 0, p)
+            : launch(ctx, q4_gemm_kernel<NTW, false>, grid, dim3(256), 0, p);
+    if (launched != hipSuccess)
+        return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);
+    if (p.splits > 1u) {
+        const size_t total = (size_t)a.M * w.N;
+        launched = launch(ctx, q4_gemm_reduce_kernel, dim3((uint32_t)((total + 255u) / 256u)),
+                          dim3(256), 0, p);
+        if (launched != hipSuccess)
+            return fail_hip(launched, "q4 gemm reduce launch", error, error_capacity);
+    }
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q
