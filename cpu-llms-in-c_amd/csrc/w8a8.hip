@@ -1,0 +1,342 @@
+// W8A8 linear: per-token symmetric int8 activations times per-output-row
+// symmetric int8 weights, int32 accumulation on v_mfma_i32_16x16x64_i8, fp32
+// rescale.  Follows the reference's quantize_i8 / q8_i8_dot / matrix_i8_rows
+// (models/minimind-o/targets/generic/minimindo_audio_encoder.c:138-306):
+//   scale = max|x| / 127, inverse = 1 / scale, q = (int8) round_half_even(x * inverse)
+//   acc[p][n] = sum_k w[n][k] * q[p][k]                         (int32, exact)
+//   out[p][n] = ((float)acc * wscale[n]) * xscale[p] + bias[n]  (fp32, left to right)
+// Integer sums do not depend on their order, so the accumulators are bit-exact
+// whatever the work split; the fp32 epilogue keeps the reference's operation
+// order and is compiled without multiply-add contraction.
+#include "device_util.h"
+#include "internal.h"
+
+#include <cstring>
+#include <new>
+
+struct mi355q_w8a8_weight {
+    mi355q_context *ctx;
+    uint4 *tiles;   // [NT][KS][64] : lane (r, kq) of tile holds w[16*tile + r][64*ks + 16*kq .. +15]
+    float *scales;  // [N]
+    uint32_t N, K, NT, KS;
+};
+
+namespace mi355q {
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+
+// rows: [N][4 + K] bytes = fp32 scale then K int8 (the MMOSENS1 Q8 tensor payload,
+// minimindo_audio_encoder.c:90,216-217).  One thread per destination uint4.
+__global__ void __launch_bounds__(256)
+w8a8_repack_kernel(const uint8_t *__restrict__ rows, uint4 *__restrict__ tiles,
+                   float *__restrict__ scales, uint32_t N, uint32_t K, uint32_t NT, uint32_t KS)
+{
+    const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)NT * KS * 64u;
+    if (index < N) {
+        // the record is only byte aligned: assemble the scale from bytes
+        const uint8_t *record = rows + index * (size_t)(4u + K);
+        uint32_t bits = record[0] | (record[1] << 8) | (record[2] << 16) | ((uint32_t)record[3] << 24);
+        scales[index] = __builtin_bit_cast(float, bits);
+    }
+    if (index >= total) return;
+    const uint32_t lane = (uint32_t)(index & 63u);
+    const size_t tile_ks = index >> 6;
+    const uint32_t ks = (uint32_t)(tile_ks % KS), tile = (uint32_t)(tile_ks / KS);
+    const uint32_t n = tile * 16u + (lane & 15u);
+    const uint32_t k0 = ks * 64u + (lane >> 4) * 16u;
+    uint32_t words[4] = {0u, 0u, 0u, 0u};
+    if (n < N) {
+        const uint8_t *source = rows + (size_t)n * (4u + K) + 4u;
+        for (uint32_t b = 0; b < 16u; ++b)
+            if (k0 + b < K) words[b >> 2] |= (uint32_t)source[k0 + b] << (8u * (b & 3u));
+    }
+    tiles[index] = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+// One workgroup per activation row: absmax, then the codes.
+__global__ void __launch_bounds__(256)
+quantize_i8_kernel(const float *__restrict__ x, uint32_t K, int8_t *__restrict__ q,
+                   float *__restrict__ scales)
+{
+    __shared__ float wave_max[4];
+    const float *row = x + (size_t)blockIdx.x * K;
+    int8_t *out = q + (size_t)blockIdx.x * K;
+    float maximum = 0.0f;
+    for (uint32_t k = threadIdx.x; k < K; k += 256u) maximum = fmaxf(maximum, fabsf(row[k]));
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1)
+        maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+    if ((threadIdx.x & 63u) == 0u) wave_max[threadIdx.x >> 6] = maximum;
+    __syncthreads();
+    maximum = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    if (!(maximum > 0.0f)) {  // all zero (or NaN-free empty) row: zero codes, scale 0
+        for (uint32_t k = threadIdx.x; k < K; k += 256u) out[k] = 0;
+        if (threadIdx.x == 0) scales[blockIdx.x] = 0.0f;
+        return;
+    }
+    const float scale = maximum / 127.0f;  // IEEE division, as the reference's
+    const float inverse = 1.0f / scale;
+    for (uint32_t k = threadIdx.x; k < K; k += 256u)
+        out[k] = (int8_t)(int)__builtin_rintf(row[k] * inverse);  // round half to even
+    if (threadIdx.x == 0) scales[blockIdx.x] = scale;
+}
+
+struct W8a8Params {
+    const uint4 *tiles;
+    const float *wscales;
+    const int8_t *q;       // [M][K]
+    const float *xscales;  // [M]
+    const float *bias;     // [N] or null
+    float *out;            // [M][N]
+    int32_t *acc;          // [M][N] or null
+    uint32_t M, N, K, NT, KS;
+};
+
+// A workgroup of four waves owns one tile of 16 weight rows and MB*16 activation
+// rows; the waves split the 64-column steps (wave w: steps w, w+4, ...) and add
+// their int32 partial sums through LDS.
+template <int MB>
+__global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
+{
+    __shared__ int red[4][MB][4][64];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15u, kq = lane >> 4;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t m0 = blockIdx.y * (MB * 16u);
+
+    intx4 acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) acc[i] = intx4{0, 0, 0, 0};
+    const uint4 *tile_words = p.tiles + (size_t)tile * p.KS * 64u + lane;
+    for (uint32_t ks = wave; ks < p.KS; ks += 4u) {
+        const intx4 b = __builtin_bit_cast(intx4, tile_words[(size_t)ks * 64u]);
+        const uint32_t k = ks * 64u + kq * 16u;
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+            const uint32_t m = m0 + 16u * i + r;
+            uint4 a = make_uint4(0u, 0u, 0u, 0u);
+            if (m < p.M && k < p.K) a = *(const uint4 *)(p.q + (size_t)m * p.K + k);
+            acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), b, acc[i],
+                                                           0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[wave][i][j][lane] = acc[i][j];
+    __syncthreads();
+    // lane (r, kq) of fragment i holds activation rows 16*i + 4*kq + j, weight row 16*tile + r
+    for (uint32_t e = threadIdx.x; e < MB * 4u * 64u; e += 256u) {
+        const uint32_t l = e & 63u, j = (e >> 6) & 3u, i = e >> 8;
+        const int sum = red[0][i][j][l] + red[1][i][j][l] + red[2][i][j][l] + red[3][i][j][l];
+        const uint32_t m = m0 + 16u * i + 4u * (l >> 4) + j;
+        const uint32_t n = tile * 16u + (l & 15u);
+        if (m >= p.M || n >= p.N) continue;
+        const size_t at = (size_t)m * p.N + n;
+        if (p.acc) p.acc[at] = sum;
+        {
+#pragma clang fp contract(off)
+            float value = (float)sum * p.wscales[n];
+            value = value * p.xscales[m];
+            value = value + (p.bias ? p.bias[n] : 0.0f);
+            p.out[at] = value;
+        }
+    }
+}
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" {
+
+int mi355q_w8a8_weight_prepare(mi355q_context *ctx, const void *rows_with_scale, uint32_t N,
+                               uint32_t K, uint32_t flags, mi355q_w8a8_weight **out, char *error,
+                               size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    if (ctx == nullptr || out == nullptr || rows_with_scale == nullptr) {
+        set_error(error, error_capacity, "w8a8_weight_prepare: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (N == 0 || K == 0 || K % 16u != 0) {
+        set_error(error, error_capacity,
+                  "w8a8_weight_prepare: shape %u x %u (columns must be a non-zero multiple of 16)", N, K);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    mi355q_w8a8_weight *weight = new (std::nothrow) mi355q_w8a8_weight();
+    if (weight == nullptr) {
+        set_error(error, error_capacity, "w8a8_weight_prepare: out of host memory");
+        return MI355Q_ERROR_RUNTIME;
+    }
+    memset(weight, 0, sizeof *weight);
+    weight->ctx = ctx;
+    weight->N = N;
+    weight->K = K;
+    weight->NT = (N + 15u) / 16u;
+    weight->KS = (K + 63u) / 64u;
+    const size_t image_bytes = (size_t)N * (4u + K);
+    const size_t items = (size_t)weight->NT * weight->KS * 64u;
+    void *staging = nullptr;
+    const uint8_t *source = (const uint8_t *)rows_with_scale;
+    hipError_t status = hipMalloc((void **)&weight->tiles, items * sizeof(uint4));
+    if (status == hipSuccess) status = hipMalloc((void **)&weight->scales, (size_t)N * sizeof(float));
+    if (status == hipSuccess && !(flags & MI355Q_SOURCE_DEVICE)) {
+        status = hipMalloc(&staging, image_bytes);
+        if (status == hipSuccess)
+            status = hipMemcpyAsync(staging, rows_with_scale, image_bytes, hipMemcpyHostToDevice,
+                                    ctx->stream);
+        source = (const uint8_t *)staging;
+    }
+    if (status == hipSuccess) {
+        const size_t threads = items > N ? items : N;
+        hipLaunchKernelGGL(w8a8_repack_kernel, dim3((uint32_t)((threads + 255u) / 256u)), dim3(256), 0,
+                           ctx->stream, source, weight->tiles, weight->scales, N, K, weight->NT,
+                           weight->KS);
+        status = hipGetLastError();
+    }
+    if (status == hipSuccess) status = hipStreamSynchronize(ctx->stream);
+    if (staging) (void)hipFree(staging);
+    if (status != hipSuccess) {
+        int code = fail_hip(status, "w8a8_weight_prepare", error, error_capacity);
+        mi355q_w8a8_weight_destroy(weight);
+        return code;
+    }
+    *out = weight;
+    return MI355Q_OK;
+}
+
+void mi355q_w8a8_weight_destroy(mi355q_w8a8_weight *weight)
+{
+    if (weight == nullptr) return;
+    if (weight->ctx) {
+        (void)hipSetDevice(weight->ctx->device);
+        (void)hipStreamSynchronize(weight->ctx->stream);
+    }
+    if (weight->tiles) (void)hipFree(weight->tiles);
+    if (weight->scales) (void)hipFree(weight->scales);
+    delete weight;
+}
+
+int mi355q_quantize_i8(mi355q_context *ctx, const float *x, uint32_t M, uint32_t K, int8_t *q,
+                       float *scales, uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || x == nullptr || q == nullptr || scales == nullptr || M == 0 || K == 0) {
+        set_error(error, error_capacity, "quantize_i8: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const bool device = (flags & MI355Q_X_DEVICE) && (flags & MI355Q_Y_DEVICE);
+    if (!device && (flags & (MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC))) {
+        set_error(error, error_capacity, "quantize_i8: pointers must be all host or all device");
+        return MI355Q_ERROR_INVALID;
+    }
+    const size_t x_bytes = (size_t)M * K * sizeof(float), q_bytes = (size_t)M * K;
+    const float *x_dev = x;
+    int8_t *q_dev = q;
+    float *s_dev = scales;
+    if (!device) {
+        int status = ensure_stage(ctx, 0, x_bytes, error, error_capacity);
+        if (status == MI355Q_OK) status = ensure_stage(ctx, 1, q_bytes + (size_t)M * 4u + 16u, error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[0], x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "activation upload");
+        x_dev = (const float *)ctx->stage[0];
+        q_dev = (int8_t *)ctx->stage[1];
+        s_dev = (float *)((char *)ctx->stage[1] + ((q_bytes + 15u) & ~(size_t)15u));
+    }
+    hipError_t launched = launch(ctx, quantize_i8_kernel, dim3(M), dim3(256), 0, x_dev, K, q_dev, s_dev);
+    if (launched != hipSuccess) return fail_hip(launched, "quantize_i8 launch", error, error_capacity);
+    if (!device) {
+        MI355Q_HIP(hipMemcpyAsync(q, q_dev, q_bytes, hipMemcpyDeviceToHost, ctx->stream), "code download");
+        MI355Q_HIP(hipMemcpyAsync(scales, s_dev, (size_t)M * 4u, hipMemcpyDeviceToHost, ctx->stream),
+                   "scale download");
+    }
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "quantize_i8 sync");
+    return MI355Q_OK;
+}
+
+int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, const int8_t *q,
+                       const float *x_scales, uint32_t M, const float *bias, float *out,
+                       int32_t *acc, uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || q == nullptr || x_scales == nullptr || out == nullptr ||
+        M == 0) {
+        set_error(error, error_capacity, "w8a8_linear: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "w8a8_linear: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    const bool device = (flags & MI355Q_X_DEVICE) && (flags & MI355Q_Y_DEVICE);
+    if (!device && (flags & (MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC))) {
+        set_error(error, error_capacity, "w8a8_linear: pointers must be all host or all device");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (device && ((uintptr_t)q & 15u) != 0) {
+        set_error(error, error_capacity, "w8a8_linear: device codes must be 16-byte aligned");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const uint32_t N = weight->N, K = weight->K;
+    const size_t q_bytes = ((size_t)M * K + 15u) & ~(size_t)15u, s_bytes = (size_t)M * 4u;
+    const size_t b_bytes = (size_t)N * 4u, o_bytes = (size_t)M * N * 4u;
+    W8a8Params p;
+    memset(&p, 0, sizeof p);
+    p.tiles = weight->tiles;
+    p.wscales = weight->scales;
+    p.q = q;
+    p.xscales = x_scales;
+    p.bias = bias;
+    p.out = out;
+    p.acc = acc;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.NT = weight->NT;
+    p.KS = weight->KS;
+    if (!device) {
+        int status = ensure_stage(ctx, 0, q_bytes + ((s_bytes + 15u) & ~(size_t)15u) + b_bytes, error,
+                                  error_capacity);
+        if (status == MI355Q_OK) status = ensure_stage(ctx, 1, 2u * o_bytes, error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        char *in = (char *)ctx->stage[0];
+        MI355Q_HIP(hipMemcpyAsync(in, q, (size_t)M * K, hipMemcpyHostToDevice, ctx->stream), "code upload");
+        p.q = (const int8_t *)in;
+        in += q_bytes;
+        MI355Q_HIP(hipMemcpyAsync(in, x_scales, s_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "scale upload");
+        p.xscales = (const float *)in;
+        in += (s_bytes + 15u) & ~(size_t)15u;
+        if (bias) {
+            MI355Q_HIP(hipMemcpyAsync(in, bias, b_bytes, hipMemcpyHostToDevice, ctx->stream),
+                       "bias upload");
+            p.bias = (const float *)in;
+        }
+        p.out = (float *)ctx->stage[1];
+        p.acc = acc ? (int32_t *)((char *)ctx->stage[1] + o_bytes) : nullptr;
+    }
+    hipError_t launched;
+    if (M > 32u)
+        launched = launch(ctx, w8a8_kernel<4>, dim3(weight->NT, (M + 63u) / 64u), dim3(256), 0, p);
+    else if (M > 16u)
+        launched = launch(ctx, w8a8_kernel<2>, dim3(weight->NT, 1), dim3(256), 0, p);
+    else
+        launched = launch(ctx, w8a8_kernel<1>, dim3(weight->NT, 1), dim3(256), 0, p);
+    if (launched != hipSuccess) return fail_hip(launched, "w8a8 kernel launch", error, error_capacity);
+    if (!device) {
+        MI355Q_HIP(hipMemcpyAsync(out, p.out, o_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                   "output download");
+        if (acc)
+            MI355Q_HIP(hipMemcpyAsync(acc, p.acc, o_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                       "accumulator download");
+    }
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "w8a8_linear sync");
+    return MI355Q_OK;
+}
+
+}  // extern "C"

@@ -67,6 +67,10 @@ SIGNATURES = {
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_sequence": (_int, [_vp, _c.POINTER(Q4Call), _sz, *_err]),
+    "mi355q_w8a8_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _u32, _c.POINTER(_vp), *_err]),
+    "mi355q_w8a8_weight_destroy": (None, [_vp]),
+    "mi355q_quantize_i8": (_int, [_vp, _vp, _u32, _u32, _vp, _vp, _u32, *_err]),
+    "mi355q_w8a8_linear": (_int, [_vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _u32, *_err]),
     "mi355q_synth_normal_f32": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_synth_normal_f16": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_quantize_q4_affine": (_int, [_vp, _u32, _u32, _int, _vp, _vp, _vp]),
@@ -232,6 +236,33 @@ class Context:
         flags = X_DEVICE | Y_DEVICE | RESIDUAL_DEVICE | (ASYNC if asynchronous else 0)
         _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, x_ptr, x_dtype, M, y_ptr,
               y_dtype, residual_ptr, residual_dtype, flags)
+
+    # ---- W8A8 ----
+    def w8a8_prepare(self, rows: np.ndarray, N: int, K: int):
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_w8a8_weight_prepare, self.handle, _ptr(rows), N, K, 0, ctypes.byref(out))
+        return out
+
+    def w8a8_destroy(self, weight):
+        self.lib.mi355q_w8a8_weight_destroy(weight)
+
+    def quantize_i8(self, x: np.ndarray):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        M, K = x.shape
+        q = np.empty((M, K), dtype=np.int8)
+        scales = np.empty(M, dtype=np.float32)
+        _call(self.lib.mi355q_quantize_i8, self.handle, _ptr(x), M, K, _ptr(q), _ptr(scales), 0)
+        return q, scales
+
+    def w8a8_linear(self, weight, N: int, q: np.ndarray, x_scales: np.ndarray, bias=None):
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        M = q.shape[0]
+        out = np.empty((M, N), dtype=np.float32)
+        acc = np.empty((M, N), dtype=np.int32)
+        _call(self.lib.mi355q_w8a8_linear, self.handle, weight, _ptr(q),
+              _ptr(np.ascontiguousarray(x_scales, dtype=np.float32)), M, _ptr(bias), _ptr(out),
+              _ptr(acc), 0)
+        return out, acc
 
     def q4_sequence(self, calls):
         """calls: a ctypes array of Q4Call (build once, reuse)."""

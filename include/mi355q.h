@@ -184,6 +184,40 @@ typedef struct {
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,
                               size_t count, char *error, size_t error_capacity);
 
+/* ---- W8A8: per-token int8 activations x per-output-row int8 weights ---------
+ *
+ * rows_with_scale: [N][4 + K] bytes, each row an fp32 scale followed by K int8
+ * weights — the Q8 tensor payload of the MMOSENS1 image
+ * (minimindo_audio_encoder.c:90,216-217; written by
+ * compiler/compile_minimindo_sensevoice_image.py:38-46).  K must be a non-zero
+ * multiple of 16.  Replaces the tensor lookup `row()` for the GPU path. */
+int mi355q_w8a8_weight_prepare(mi355q_context *ctx, const void *rows_with_scale,
+                               uint32_t N, uint32_t K, uint32_t flags,
+                               mi355q_w8a8_weight **out,
+                               char *error, size_t error_capacity);
+void mi355q_w8a8_weight_destroy(mi355q_w8a8_weight *weight);
+
+/* Per-token symmetric quantization of x[M][K] (fp32): scales[m] = max|x[m]|/127,
+ * q = (int8) round_half_even(x * (1/scale)); an all-zero row gives zero codes
+ * and scale 0.  Bit-exact with quantize_i8 / quantize_sequence_i8
+ * (minimindo_audio_encoder.c:186-215,291-297).  flags: 0 for host pointers, or
+ * MI355Q_X_DEVICE|MI355Q_Y_DEVICE (x, q and scales all on the device),
+ * optionally with MI355Q_ASYNC. */
+int mi355q_quantize_i8(mi355q_context *ctx, const float *x, uint32_t M, uint32_t K,
+                       int8_t *q, float *scales, uint32_t flags,
+                       char *error, size_t error_capacity);
+
+/* out[m][n] = ((float)acc[m][n] * weight_scale[n]) * x_scales[m] + bias[n], with
+ * acc[m][n] = sum_k w[n][k] * q[m][k] in int32; bias may be NULL; when `acc` is
+ * not NULL the int32 accumulators are written there as well.  Replaces
+ * matrix_sequence_i8_quantized (minimindo_audio_encoder.c:267-306): same
+ * argument meaning, position-major fp32 output.  flags as for
+ * mi355q_quantize_i8 (all pointers host, or all device). */
+int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight,
+                       const int8_t *q, const float *x_scales, uint32_t M,
+                       const float *bias, float *out, int32_t *acc, uint32_t flags,
+                       char *error, size_t error_capacity);
+
 #ifdef __cplusplus
 }
 #endif

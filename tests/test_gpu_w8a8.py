@@ -1,0 +1,84 @@
+"""GPU parity of the W8A8 path against the CPU oracle and the reference's golden vectors:
+int8 codes, scales, int32 accumulators and fp32 outputs must all be bit-exact."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).resolve().parent / "golden" / "w8a8_minimindo.npz"
+
+
+def check(engine, oracle, gpu, M, K, N, seed, bias=True):
+    x = engine.synth_normal_f32(seed, 1.0, M * K).reshape(M, K)
+    rows = engine.synth_w8_rows(seed + 1, 0.02, N, K)
+    b = engine.synth_normal_f32(seed + 2, 1.0, N) if bias else None
+    print(f"w8a8 case M={M} K={K} N={N} bias={bias}", flush=True)
+    q, scales = gpu.quantize_i8(x)
+    q_ref, s_ref = oracle.quantize_i8(x)
+    assert np.array_equal(q, q_ref)
+    assert np.array_equal(scales.view(np.uint32), s_ref.view(np.uint32))
+    weight = gpu.w8a8_prepare(rows, N, K)
+    try:
+        out, acc = gpu.w8a8_linear(weight, N, q, scales, b)
+    finally:
+        gpu.w8a8_destroy(weight)
+    out_ref, acc_ref = oracle.w8a8_linear(rows, N, K, q_ref, s_ref, b)
+    assert acc.tobytes() == acc_ref.tobytes()          # the memcmp gate on the int32 accumulators
+    assert np.array_equal(out.view(np.uint32), out_ref.view(np.uint32))
+
+
+def test_config5(engine, oracle, gpu):
+    """BASELINE config 5: M=64, K=1024, N=4096."""
+    check(engine, oracle, gpu, 64, 1024, 4096, 31)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 16, 16), (3, 48, 20), (17, 560, 100), (40, 512, 2048),
+                                   (130, 2048, 512), (64, 1024, 4100)])
+def test_shapes(engine, oracle, gpu, M, K, N):
+    check(engine, oracle, gpu, M, K, N, 7 + M, bias=(M % 2 == 0))
+
+
+def test_reference_golden_vectors(engine, gpu):
+    g = np.load(GOLDEN, allow_pickle=False)
+    x, rows, bias = g["x"], g["rows"], g["bias"]
+    N, K = g["w"].shape
+    q, scales = gpu.quantize_i8(x)
+    assert np.array_equal(q, g["q"]) and np.array_equal(scales.view(np.uint32), g["scales"].view(np.uint32))
+    weight = gpu.w8a8_prepare(rows, N, K)
+    try:
+        out, acc = gpu.w8a8_linear(weight, N, q, scales, bias)
+        out2, _ = gpu.w8a8_linear(weight, N, q, scales, None)
+    finally:
+        gpu.w8a8_destroy(weight)
+    assert np.array_equal(acc, g["dots"])
+    assert np.array_equal(out.view(np.uint32), g["out_bias"].view(np.uint32))
+    assert np.array_equal(out2.view(np.uint32), g["out_nobias"].view(np.uint32))
+
+
+def test_saturating_inputs_keep_int32_exact(engine, oracle, gpu):
+    """+-127 codes against +-127 weights at K=2048: |acc| = 33,032,192 > 2^24, still exact in int32."""
+    M, K, N = 16, 2048, 32
+    x = np.ones((M, K), dtype=np.float32)
+    x[1::2] *= -1
+    w = np.ones((N, K), dtype=np.float32) * 0.5
+    w[::3] *= -1
+    rows = np.empty(N * (4 + K), dtype=np.uint8)
+    assert engine.library().mi355q_quantize_w8_rows(w.ctypes.data, N, K, rows.ctypes.data) == 0
+    q, scales = gpu.quantize_i8(x)
+    assert set(np.unique(q)) == {-127, 127}
+    weight = gpu.w8a8_prepare(rows, N, K)
+    try:
+        out, acc = gpu.w8a8_linear(weight, N, q, scales, None)
+    finally:
+        gpu.w8a8_destroy(weight)
+    assert np.max(np.abs(acc)) == 127 * 127 * K
+    out_ref, acc_ref = oracle.w8a8_linear(rows, N, K, q, scales, None)
+    assert np.array_equal(acc, acc_ref) and np.array_equal(out.view(np.uint32), out_ref.view(np.uint32))
+
+
+def test_argument_errors(engine, gpu):
+    rows = engine.synth_w8_rows(1, 0.02, 16, 24)
+    with pytest.raises(engine.Mi355qError) as info:
+        gpu.w8a8_prepare(rows, 16, 24)  # 24 is not a multiple of 16
+    assert info.value.status == engine.ERROR_INVALID
