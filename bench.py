@@ -6,7 +6,8 @@ decoder layer at M=1 — q 5120->6144, k and v 5120->1024, o 6144->5120, gate an
 up 5120->17408, down 17408->5120 — in affine-Q4 group-64 with bf16 scale/bias,
 fp16 activations and fp16 outputs, on seeded synthetic weights (N(0,0.02)
 before quantization) and activations (N(0,1)).  One step is one pass over the
-seven linears of one weight copy; successive steps rotate over `--copies`
+seven linears of one weight copy (four launches: q|k|v and gate|up share their
+activations and go out as one launch each, then o and down); successive steps rotate over `--copies`
 distinct prepared copies (>= 1.5 GB in total) so that the 256 MB memory-side
 cache cannot serve the weights and the figure is an HBM figure.
 
@@ -53,7 +54,7 @@ def q4_bytes(N, K, M, y_bytes=2):
     return N * K // 2 + N * (K // 64) * 4 + M * K * 2 + M * N * y_bytes
 
 
-def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose):
+def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True):
     """Prepares `copies` device copies of every matrix plus activations/outputs."""
     x_ptr, y_ptr, weights, host = {}, {}, [[] for _ in range(copies)], {}
     for index, (name, N, K) in enumerate(shapes):
@@ -72,9 +73,17 @@ def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose):
                   file=sys.stderr, flush=True)
     calls = []
     for copy in range(copies):
-        items = [(weights[copy][i], x_ptr[K], engine.F16, M, y_ptr[name], engine.F16)
-                 for i, (name, N, K) in enumerate(shapes)]
-        calls.append(engine.make_calls(items))
+        # linears that read the same activations go out as one launch (q|k|v, gate|up)
+        groups = []
+        for i, (name, N, K) in enumerate(shapes):
+            target = (weights[copy][i], y_ptr[name])
+            share = fuse and groups and groups[-1][1] == K and name.split("_")[0] in ("k", "v", "up")
+            if share:
+                groups[-1][0].append(target)
+            else:
+                groups.append(([target], K))
+        calls.append(engine.make_calls([(targets, x_ptr[K], engine.F16, M, engine.F16)
+                                        for targets, K in groups]))
     return calls, weights, host, x_ptr, y_ptr
 
 
@@ -111,6 +120,8 @@ def main():
     parser.add_argument("--copies", type=int, default=8)
     parser.add_argument("--rows", type=int, default=1, help="activation rows M (1..8)")
     parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1"])
+    parser.add_argument("--unfused", action="store_true",
+                        help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
     parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args()
@@ -128,7 +139,8 @@ def main():
     ctx = engine.Context(0)  # raises without a GPU
     info = ctx.info()
     calls, weights, host, x_ptr, y_ptr = build_workload(engine, ctx, shapes, M, copies, meta_kind,
-                                                        args.verbose)
+                                                        args.verbose, fuse=not args.unfused)
+    launches_per_step = len(calls[0])
     step_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
 
     def run_steps(count):
@@ -151,10 +163,10 @@ def main():
 
     # measured plain-read ceiling: whole 2 GiB pass, and launches the size of one weight matrix
     read_long = ctx.probe_read_bandwidth(2 << 30, 3, 1, 0)
-    read_short = ctx.probe_read_bandwidth(2 << 30, 3, 1, int(step_bytes / len(shapes)))
+    read_short = ctx.probe_read_bandwidth(2 << 30, 3, 1, int(step_bytes / launches_per_step))
 
     value = step_bytes * args.steps / wall / 1e9
-    bytes_per_launch = step_bytes / len(shapes)
+    bytes_per_launch = step_bytes / launches_per_step
     avg_kernel_us = kernel_ms * 1e3 / max(launches, 1)
     achieved = bytes_per_launch / (avg_kernel_us * 1e-6) / 1e9
     result = {
@@ -177,6 +189,7 @@ def main():
                          "g64, bf16 scale+bias, fp16 x and y" % M) if args.workload == "layer_m1"
                         else "affine-Q4 g64 GEMV K=1024 N=3584 M=%d, fp16 scale+bias, fp16 x and y" % M,
             "linears_per_step": len(shapes),
+            "launches_per_step": launches_per_step,
             "algorithmic_bytes_per_step": step_bytes,
             "weight_copies_rotated": copies,
             "rotated_bytes": step_bytes * copies,

@@ -364,26 +364,42 @@ size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight)
     return weight ? weight->image_bytes : 0;
 }
 
-int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const void *x,
-                     int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,
-                     int residual_dtype, uint32_t flags, char *error, size_t error_capacity)
+int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count,
+                           const void *x, int x_dtype, uint32_t M, int y_dtype, int residual_dtype,
+                           uint32_t flags, char *error, size_t error_capacity)
 {
-    if (ctx == nullptr || weight == nullptr || x == nullptr || y == nullptr) {
-        set_error(error, error_capacity, "q4_linear: null argument");
+    if (ctx == nullptr || targets == nullptr || x == nullptr || count == 0 || count > kMaxTargets) {
+        set_error(error, error_capacity, "q4_linear: null argument or target count outside 1..%u",
+                  kMaxTargets);
         return MI355Q_ERROR_INVALID;
     }
-    if (weight->ctx != ctx) {
-        set_error(error, error_capacity, "q4_linear: weight belongs to another context");
-        return MI355Q_ERROR_INVALID;
+    bool any_residual = false;
+    for (uint32_t t = 0; t < count; ++t) {
+        const mi355q_q4_target &target = targets[t];
+        if (target.weight == nullptr || target.y == nullptr) {
+            set_error(error, error_capacity, "q4_linear: null weight or output (target %u)", t);
+            return MI355Q_ERROR_INVALID;
+        }
+        if (target.weight->ctx != ctx) {
+            set_error(error, error_capacity, "q4_linear: weight belongs to another context");
+            return MI355Q_ERROR_INVALID;
+        }
+        if (target.weight->dev.K != targets[0].weight->dev.K ||
+            target.weight->dev.meta_kind != targets[0].weight->dev.meta_kind) {
+            set_error(error, error_capacity,
+                      "q4_linear: weights of one call must share K and the metadata kind");
+            return MI355Q_ERROR_INVALID;
+        }
+        any_residual = any_residual || target.residual != nullptr;
     }
     if (M == 0 || !dtype_valid(x_dtype) || !dtype_valid(y_dtype) ||
-        (residual != nullptr && !dtype_valid(residual_dtype))) {
+        (any_residual && !dtype_valid(residual_dtype))) {
         set_error(error, error_capacity, "q4_linear: M=%u x_dtype=%d y_dtype=%d residual_dtype=%d",
                   M, x_dtype, y_dtype, residual_dtype);
         return MI355Q_ERROR_INVALID;
     }
     const bool x_dev = flags & MI355Q_X_DEVICE, y_dev = flags & MI355Q_Y_DEVICE;
-    const bool r_dev = residual == nullptr || (flags & MI355Q_RESIDUAL_DEVICE);
+    const bool r_dev = !any_residual || (flags & MI355Q_RESIDUAL_DEVICE);
     if ((flags & MI355Q_ASYNC) && !(x_dev && y_dev && r_dev)) {
         set_error(error, error_capacity, "q4_linear: ASYNC needs device pointers throughout");
         return MI355Q_ERROR_INVALID;
@@ -393,19 +409,26 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const 
         return MI355Q_ERROR_INVALID;
     }
     MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
-    const Q4Device &dev = weight->dev;
-    const size_t x_bytes = (size_t)M * dev.K * dtype_bytes(x_dtype);
-    const size_t y_bytes = (size_t)M * dev.N * dtype_bytes(y_dtype);
-    const size_t r_bytes = residual ? (size_t)M * dev.N * dtype_bytes(residual_dtype) : 0;
+    const uint32_t K = targets[0].weight->dev.K;
+    const size_t x_bytes = (size_t)M * K * dtype_bytes(x_dtype);
+    // host outputs / residuals are staged back to back, each 256-byte aligned
+    size_t y_offset[kMaxTargets], r_offset[kMaxTargets], y_total = 0, r_total = 0;
+    for (uint32_t t = 0; t < count; ++t) {
+        const size_t cells = (size_t)M * targets[t].weight->dev.N;
+        y_offset[t] = y_total;
+        y_total += (cells * dtype_bytes(y_dtype) + 255u) & ~(size_t)255u;
+        r_offset[t] = r_total;
+        if (targets[t].residual) r_total += (cells * dtype_bytes(residual_dtype) + 255u) & ~(size_t)255u;
+    }
 
     Q4LinearArgs args;
+    memset(&args, 0, sizeof args);
     args.x = x;
     args.x_dtype = x_dtype;
     args.M = M;
-    args.y = y;
     args.y_dtype = y_dtype;
-    args.residual = residual;
     args.residual_dtype = residual_dtype;
+    args.count = count;
     int status;
     if (!x_dev) {
         if ((status = ensure_stage(ctx, 0, x_bytes, error, error_capacity)) != MI355Q_OK) return status;
@@ -413,32 +436,52 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const 
                    "activation upload");
         args.x = ctx->stage[0];
     }
-    if (!y_dev) {
-        if ((status = ensure_stage(ctx, 1, y_bytes, error, error_capacity)) != MI355Q_OK) return status;
-        args.y = ctx->stage[1];
-    }
-    if (!r_dev) {
-        if ((status = ensure_stage(ctx, 2, r_bytes, error, error_capacity)) != MI355Q_OK) return status;
-        MI355Q_HIP(hipMemcpyAsync(ctx->stage[2], residual, r_bytes, hipMemcpyHostToDevice,
-                                  ctx->stream),
-                   "residual upload");
-        args.residual = ctx->stage[2];
+    if (!y_dev && (status = ensure_stage(ctx, 1, y_total, error, error_capacity)) != MI355Q_OK)
+        return status;
+    if (!r_dev && (status = ensure_stage(ctx, 2, r_total, error, error_capacity)) != MI355Q_OK)
+        return status;
+    for (uint32_t t = 0; t < count; ++t) {
+        const size_t cells = (size_t)M * targets[t].weight->dev.N;
+        args.targets[t].w = &targets[t].weight->dev;
+        args.targets[t].y = y_dev ? targets[t].y : (void *)((char *)ctx->stage[1] + y_offset[t]);
+        args.targets[t].residual = targets[t].residual;
+        if (targets[t].residual && !r_dev) {
+            void *staged = (char *)ctx->stage[2] + r_offset[t];
+            MI355Q_HIP(hipMemcpyAsync(staged, targets[t].residual, cells * dtype_bytes(residual_dtype),
+                                      hipMemcpyHostToDevice, ctx->stream),
+                       "residual upload");
+            args.targets[t].residual = staged;
+        }
     }
 
     const uint32_t stream_rows = x_dtype == MI355Q_F32 ? 2u * M : M;
     if (stream_rows <= 16u) {
-        status = q4_stream_linear(ctx, dev, args, error, error_capacity);
+        status = q4_stream_linear(ctx, args, error, error_capacity);
     } else {
-        status = q4_gemm_linear(ctx, dev, args, error, error_capacity);
+        status = MI355Q_OK;
+        for (uint32_t t = 0; t < count && status == MI355Q_OK; ++t)
+            status = q4_gemm_linear(ctx, args, t, error, error_capacity);
     }
     if (status != MI355Q_OK) return status;
 
     if (!y_dev)
-        MI355Q_HIP(hipMemcpyAsync(y, ctx->stage[1], y_bytes, hipMemcpyDeviceToHost, ctx->stream),
-                   "output download");
+        for (uint32_t t = 0; t < count; ++t)
+            MI355Q_HIP(hipMemcpyAsync(targets[t].y, args.targets[t].y,
+                                      (size_t)M * targets[t].weight->dev.N * dtype_bytes(y_dtype),
+                                      hipMemcpyDeviceToHost, ctx->stream),
+                       "output download");
     if (!(flags & MI355Q_ASYNC))
         MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear sync");
     return MI355Q_OK;
+}
+
+int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const void *x,
+                     int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,
+                     int residual_dtype, uint32_t flags, char *error, size_t error_capacity)
+{
+    mi355q_q4_target target = {weight, y, residual};
+    return mi355q_q4_linear_multi(ctx, &target, 1, x, x_dtype, M, y_dtype, residual_dtype, flags, error,
+                                  error_capacity);
 }
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,
@@ -452,8 +495,8 @@ int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, 
     for (size_t i = 0; i < count; ++i) {
         const mi355q_q4_call &c = calls[i];
         char inner[256] = "";
-        int status = mi355q_q4_linear(ctx, c.weight, c.x, c.x_dtype, c.M, c.y, c.y_dtype,
-                                      c.residual, c.residual_dtype, flags, inner, sizeof inner);
+        int status = mi355q_q4_linear_multi(ctx, c.targets, c.target_count, c.x, c.x_dtype, c.M,
+                                            c.y_dtype, c.residual_dtype, flags, inner, sizeof inner);
         if (status != MI355Q_OK) {
             set_error(error, error_capacity, "call %zu: %s", i, inner);
             return status;

@@ -117,19 +117,25 @@ hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
                             hipStream_t stream);
 
 // q4_stream.hip
+constexpr uint32_t kMaxTargets = 4;
+struct Q4Target {
+    const Q4Device *w;
+    void *y;
+    const void *residual;
+};
+// One activation matrix against up to four weights of the same K and metadata kind.
 struct Q4LinearArgs {
     const void *x;
     int x_dtype;
     uint32_t M;
-    void *y;
     int y_dtype;
-    const void *residual;
     int residual_dtype;
+    uint32_t count;
+    Q4Target targets[kMaxTargets];
 };
-int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
-                     char *error, size_t error_capacity);
-// q4_gemm.hip
-int q4_gemm_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
-                   char *error, size_t error_capacity);
+int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity);
+// q4_gemm.hip (one target at a time: `target` selects it)
+int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
+                   size_t error_capacity);
 
 }  // namespace mi355q

@@ -204,9 +204,10 @@ q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__re
     out[index] = (_Float16)load_as_float(x, x_dtype, index);
 }
 
-int q4_gemm_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a, char *error,
+int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
                    size_t error_capacity)
 {
+    const Q4Device &w = *a.targets[target].w;
     GemmParams p;
     memset(&p, 0, sizeof p);
     p.codes = w.codes;
@@ -223,8 +224,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = (const _Float16 *)ctx->stage[3];
     }
-    p.y = a.y;
-    p.residual = a.residual;
+    p.y = a.targets[target].y;
+    p.residual = a.targets[target].residual;
     p.M = a.M;
     p.N = w.N;
     p.K = w.K;

@@ -25,12 +25,16 @@
 namespace mi355q {
 
 struct StreamParams {
-    const uint4 *codes;
-    const uint2 *meta;
+    // up to kMaxTargets weights share the activations; workgroups
+    // [first_block[t], first_block[t+1]) work on weight t
+    const uint4 *codes[kMaxTargets];
+    const uint2 *meta[kMaxTargets];
+    void *y[kMaxTargets];
+    const void *residual[kMaxTargets];
+    uint32_t N[kMaxTargets], NT[kMaxTargets], first_block[kMaxTargets];
+    uint32_t targets;
     const _Float16 *x;  // [rows][K] fp16
-    void *y;
-    const void *residual;
-    uint32_t M, N, K, NT, T;
+    uint32_t M, K, T;
     uint32_t rows;         // M, or 2*M when fp32 activations are carried as (value, remainder) pairs
     uint32_t chunks;       // column chunks (1 unless the activations overflow the LDS budget)
     uint32_t chunk_steps;  // steps per chunk (the last chunk may be shorter, never shorter than W)
@@ -55,7 +59,12 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15u;
     const uint32_t kq = lane >> 4;
-    const uint32_t tile0 = blockIdx.x * TB;
+    uint32_t target = 0;
+#pragma unroll
+    for (uint32_t t = 1; t < kMaxTargets; ++t)
+        if (t < p.targets && blockIdx.x >= p.first_block[t]) target = t;
+    const uint32_t NT = p.NT[target], N = p.N[target];
+    const uint32_t tile0 = (blockIdx.x - p.first_block[target]) * TB;
 
     uint4 *xs = lds;                                                 // [chunk octets][MP]
     float *red = (float *)(lds + (size_t)p.chunk_steps * 16u * MP);  // [W][TB][NJ][64]
@@ -67,9 +76,9 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
         uint32_t tile = tile0 + tb;
-        tile = tile < p.NT ? tile : p.NT - 1u;
-        codes_tile[tb] = p.codes + (size_t)tile * 64u + lane;
-        meta_tile[tb] = p.meta + (size_t)tile * 16u + r;
+        tile = tile < NT ? tile : NT - 1u;
+        codes_tile[tb] = p.codes[target] + (size_t)tile * 64u + lane;
+        meta_tile[tb] = p.meta[target] + (size_t)tile * 16u + r;
     }
 
     floatx4 acc[TB];
@@ -97,8 +106,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             step = step < p.T ? step : p.T - 1u;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * p.NT * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * p.NT * 16u);
+                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * NT * 64u);
+                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * NT * 16u);
             }
         };
         // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
@@ -192,7 +201,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         const uint32_t tb = e >> 6, l = e & 63u;
         const uint32_t tile = tile0 + tb;
         const uint32_t n = tile * kTileRows + (l & 15u);
-        if (tile >= p.NT || n >= p.N) continue;
+        if (tile >= NT || n >= N) continue;
         float v[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
@@ -212,9 +221,9 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 value += v[(j + 1) % NJ];
                 m = row >> 1;
             }
-            const size_t at = (size_t)m * p.N + n;
-            if (p.residual) value += load_as_float(p.residual, p.residual_dtype, at);
-            store_from_float(p.y, p.y_dtype, at, value);
+            const size_t at = (size_t)m * N + n;
+            if (p.residual[target]) value += load_as_float(p.residual[target], p.residual_dtype, at);
+            store_from_float(p.y[target], p.y_dtype, at, value);
         }
     }
 }
@@ -252,7 +261,8 @@ template <int MP, int TB, int D, int W>
 static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
 {
     constexpr int NJ = MP < 4 ? MP : 4;
-    const uint32_t blocks = (p.NT + TB - 1) / TB;
+    uint32_t blocks = 0;
+    for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
     const size_t lds = (size_t)p.chunk_steps * 16u * MP * sizeof(uint4) +
                        (size_t)W * TB * NJ * 64u * sizeof(float);
     if (p.meta_bf16)
@@ -299,7 +309,7 @@ static void choose_chunks(StreamShape &shape, uint32_t T)
     shape.chunk_steps = each;
 }
 
-static StreamShape choose_shape(const mi355q_context *ctx, const Q4Device &w, int mp)
+static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp)
 {
     StreamShape shape;
     shape.mp = mp;
@@ -308,9 +318,9 @@ static StreamShape choose_shape(const mi355q_context *ctx, const Q4Device &w, in
     // busy without queueing; more waves per workgroup when there are few tiles
     shape.tb = 1;
     shape.depth = 2;
-    const uint32_t want = (16u * cus + w.NT - 1) / w.NT;
+    const uint32_t want = (16u * cus + NT_total - 1) / NT_total;
     shape.waves = want <= 2u ? 2 : want <= 5u ? 4 : 8;
-    while (shape.waves > 2 && (uint32_t)shape.waves > w.T) shape.waves /= 2;
+    while (shape.waves > 2 && (uint32_t)shape.waves > T) shape.waves /= 2;
     const char *force = getenv("MI355Q_Q4_STREAM");  // "TB,DEPTH,WAVES" for experiments
     int ft = 0, fd = 0, fw = 0;
     if (force && sscanf(force, "%d,%d,%d", &ft, &fd, &fw) == 3) {
@@ -318,22 +328,22 @@ static StreamShape choose_shape(const mi355q_context *ctx, const Q4Device &w, in
         shape.depth = fd;
         shape.waves = fw;
     }
-    choose_chunks(shape, w.T);
+    choose_chunks(shape, T);
     // fall back to smaller workgroups when the activations crowd LDS
     if (stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps) > 64u * 1024u) {
         shape.waves = 4;
-        choose_chunks(shape, w.T);
+        choose_chunks(shape, T);
     }
     if (stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps) > 64u * 1024u) {
         shape.tb = 1;
-        choose_chunks(shape, w.T);
+        choose_chunks(shape, T);
     }
     return shape;
 }
 
-int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs &a,
-                     char *error, size_t error_capacity)
+int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity)
 {
+    const Q4Device &first = *a.targets[0].w;
     const bool pair = a.x_dtype == MI355Q_F32;
     const uint32_t rows = pair ? 2u * a.M : a.M;
     if (rows > 16u) {
@@ -345,41 +355,50 @@ int q4_stream_linear(mi355q_context *ctx, const Q4Device &w, const Q4LinearArgs 
 
     StreamParams p;
     memset(&p, 0, sizeof p);
-    p.codes = w.codes;
-    p.meta = w.meta;
     p.x = (const _Float16 *)a.x;
     if (a.x_dtype != MI355Q_F16) {
-        const size_t bytes = (size_t)rows * w.K * sizeof(_Float16);
+        const size_t bytes = (size_t)rows * first.K * sizeof(_Float16);
         int status = ensure_stage(ctx, 3, bytes, error, error_capacity);
         if (status != MI355Q_OK) return status;
-        const size_t count = (size_t)a.M * w.K;
+        const size_t count = (size_t)a.M * first.K;
         hipError_t converted =
             launch(ctx, q4_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256), 0,
-                   a.x, a.x_dtype, (_Float16 *)ctx->stage[3], a.M, w.K);
+                   a.x, a.x_dtype, (_Float16 *)ctx->stage[3], a.M, first.K);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = (const _Float16 *)ctx->stage[3];
     }
-    const StreamShape shape = choose_shape(ctx, w, mp);
-    p.y = a.y;
-    p.residual = a.residual;
+    uint32_t tiles = 0;
+    for (uint32_t t = 0; t < a.count; ++t) tiles += a.targets[t].w->NT;
+    const StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
+    uint32_t block = 0;
+    for (uint32_t t = 0; t < a.count; ++t) {
+        const Q4Device &w = *a.targets[t].w;
+        p.codes[t] = w.codes;
+        p.meta[t] = w.meta;
+        p.y[t] = a.targets[t].y;
+        p.residual[t] = a.targets[t].residual;
+        p.N[t] = w.N;
+        p.NT[t] = w.NT;
+        p.first_block[t] = block;
+        block += (w.NT + shape.tb - 1) / shape.tb;
+    }
+    p.targets = a.count;
     p.M = a.M;
-    p.N = w.N;
-    p.K = w.K;
-    p.NT = w.NT;
-    p.T = w.T;
+    p.K = first.K;
+    p.T = first.T;
     p.rows = rows;
     p.chunks = shape.chunks;
     p.chunk_steps = shape.chunk_steps;
     p.pair = pair;
     p.y_dtype = a.y_dtype;
     p.residual_dtype = a.residual_dtype;
-    p.meta_bf16 = w.meta_kind == MI355Q_META_BF16_PLANES;
+    p.meta_bf16 = first.meta_kind == MI355Q_META_BF16_PLANES;
 
     const size_t lds = stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps);
     if (lds > 64u * 1024u) {
         set_error(error, error_capacity, "q4 stream kernel: %zu bytes of LDS needed (K=%u, rows=%u)",
-                  lds, w.K, rows);
+                  lds, first.K, rows);
         return MI355Q_ERROR_INVALID;
     }
     hipError_t launched;

@@ -41,9 +41,13 @@ class DeviceInfo(_c.Structure):
     ]
 
 
+class Q4Target(_c.Structure):
+    _fields_ = [("weight", _vp), ("y", _vp), ("residual", _vp)]
+
+
 class Q4Call(_c.Structure):
-    _fields_ = [("weight", _vp), ("x", _vp), ("y", _vp), ("residual", _vp), ("M", _u32),
-                ("x_dtype", _int), ("y_dtype", _int), ("residual_dtype", _int)]
+    _fields_ = [("x", _vp), ("M", _u32), ("x_dtype", _int), ("y_dtype", _int),
+                ("residual_dtype", _int), ("target_count", _u32), ("targets", Q4Target * 4)]
 
 
 # name -> (restype, argtypes): every symbol the two headers declare
@@ -66,6 +70,8 @@ SIGNATURES = {
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
+    "mi355q_q4_linear_multi": (_int, [_vp, _c.POINTER(Q4Target), _u32, _vp, _int, _u32, _int, _int,
+                                      _u32, *_err]),
     "mi355q_q4_linear_sequence": (_int, [_vp, _c.POINTER(Q4Call), _sz, *_err]),
     "mi355q_w8a8_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_w8a8_weight_destroy": (None, [_vp]),
@@ -230,6 +236,18 @@ class Context:
               _ptr(y), y_dtype, _ptr(residual), residual_dtype, 0)
         return y
 
+    def q4_linear_multi(self, weights, x: np.ndarray, x_dtype: int, y_dtype: int = F32):
+        """Host-array form of the shared-x call: returns one y per weight."""
+        x = np.ascontiguousarray(x)
+        M = x.shape[0]
+        ys = [np.empty((M, w.N), dtype=_NP_DTYPE[y_dtype]) for w in weights]
+        targets = (Q4Target * len(weights))()
+        for slot, w, y in zip(targets, weights, ys):
+            slot.weight, slot.y, slot.residual = w.handle, y.ctypes.data, None
+        _call(self.lib.mi355q_q4_linear_multi, self.handle, targets, len(weights), _ptr(x), x_dtype, M,
+              y_dtype, F32, 0)
+        return ys
+
     def q4_linear_device(self, weight: Q4Weight, x_ptr: int, x_dtype: int, M: int, y_ptr: int,
                          y_dtype: int, residual_ptr: int | None = None,
                          residual_dtype: int = F32, asynchronous: bool = True):
@@ -270,15 +288,22 @@ class Context:
 
 
 def make_calls(items):
-    """items: iterable of (weight, x_ptr, x_dtype, M, y_ptr, y_dtype[, residual_ptr, residual_dtype])."""
+    """items: iterable of (targets, x_ptr, x_dtype, M, y_dtype[, residual_dtype]) where targets is
+    a Q4Weight with its y pointer `(weight, y_ptr[, residual_ptr])` or a list of up to four of them
+    (one launch, shared x)."""
     items = list(items)
     array = (Q4Call * len(items))()
     for slot, item in zip(array, items):
-        weight, x_ptr, x_dtype, M, y_ptr, y_dtype = item[:6]
-        slot.weight, slot.x, slot.y = weight.handle, x_ptr, y_ptr
-        slot.M, slot.x_dtype, slot.y_dtype = M, x_dtype, y_dtype
-        slot.residual = item[6] if len(item) > 6 else None
-        slot.residual_dtype = item[7] if len(item) > 7 else F32
+        targets, x_ptr, x_dtype, M, y_dtype = item[:5]
+        if isinstance(targets, tuple):
+            targets = [targets]
+        slot.x, slot.M, slot.x_dtype, slot.y_dtype = x_ptr, M, x_dtype, y_dtype
+        slot.residual_dtype = item[5] if len(item) > 5 else F32
+        slot.target_count = len(targets)
+        for index, target in enumerate(targets):
+            slot.targets[index].weight = target[0].handle
+            slot.targets[index].y = target[1]
+            slot.targets[index].residual = target[2] if len(target) > 2 else None
     return array
 
 

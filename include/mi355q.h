@@ -167,18 +167,35 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight,
                      const void *residual, int residual_dtype,
                      uint32_t flags, char *error, size_t error_capacity);
 
-/* A run of linears queued back to back on the context's stream with one host
- * call, all pointers on the device and nothing waited for — the way the
+/* One activation matrix against up to four weights that share K and the
+ * metadata kind, in ONE kernel launch for M <= 16: y_t = x * w_t^T (+ residual_t).
+ * This is how a decoder layer uses the path — q, k and v read the same x, and
+ * so do gate and up (the reference fuses them the same way: one 14336-row
+ * q|k|v matrix, qwen38_m3_attention_image.h:11-14; qwen38_q4_gate_up_silu,
+ * qwen38_q4.metal:129-151) — and it spares the small matrices their own launch.
+ * For M > 16 the targets run one after the other. */
+typedef struct {
+    const mi355q_q4_weight *weight;
+    void *y;              /* [M][N_t] of y_dtype */
+    const void *residual; /* [M][N_t] of residual_dtype, or NULL */
+} mi355q_q4_target;
+
+int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
+                           uint32_t count, const void *x, int x_dtype, uint32_t M,
+                           int y_dtype, int residual_dtype, uint32_t flags,
+                           char *error, size_t error_capacity);
+
+/* A run of (multi-)linears queued back to back on the context's stream with one
+ * host call, all pointers on the device and nothing waited for — the way the
  * reference encodes every matvec of a forward pass into one command buffer
  * before committing it (qwen38_m3_decode.m:1614-1699).  Stops at the first
  * call that fails and reports its index in the message. */
 typedef struct {
-    const mi355q_q4_weight *weight;
     const void *x;
-    void *y;
-    const void *residual; /* or NULL */
     uint32_t M;
     int x_dtype, y_dtype, residual_dtype;
+    uint32_t target_count; /* 1..4 */
+    mi355q_q4_target targets[4];
 } mi355q_q4_call;
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,

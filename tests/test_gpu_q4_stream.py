@@ -118,3 +118,33 @@ def test_argument_errors(engine, gpu):
         assert info.value.status == engine.ERROR_INVALID
     finally:
         weight.destroy()
+
+
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_shared_activation_multi_launch(engine, oracle, gpu, M):
+    """q|k|v-style call: three weights of different row counts, one launch, same x; each output
+    must equal the single-weight call bit for bit and pass the oracle gate."""
+    K = 1536
+    rows = [640, 100, 1024]
+    images = [engine.synth_q4_affine(60 + i, 0.02, N, K, engine.META_BF16_PLANES)
+              for i, N in enumerate(rows)]
+    x = make_x(engine, 70, M, K, engine.F16)
+    weights = [gpu.q4_prepare(q, a, b, N, K, engine.META_BF16_PLANES)
+               for (q, a, b), N in zip(images, rows)]
+    try:
+        print(f"multi case M={M}", flush=True)
+        together = gpu.q4_linear_multi(weights, x, engine.F16, engine.F32)
+        for (q, a, b), N, w, y in zip(images, rows, weights, together):
+            alone = gpu.q4_linear(w, x, engine.F16, engine.F32)
+            assert np.array_equal(alone.view(np.uint32), y.view(np.uint32))
+            ref = oracle.q4_linear(q, a, b, engine.META_BF16_PLANES, N, K, x, engine.F16, M)
+            assert q4_relative_error(y, ref) <= TOLERANCE
+        mixed = gpu.q4_prepare(*engine.synth_q4_affine(1, 0.02, 32, 512, engine.META_BF16_PLANES),
+                               32, 512, engine.META_BF16_PLANES)
+        with pytest.raises(engine.Mi355qError) as info:
+            gpu.q4_linear_multi([weights[0], mixed], x, engine.F16, engine.F32)
+        assert info.value.status == engine.ERROR_INVALID
+        mixed.destroy()
+    finally:
+        for w in weights:
+            w.destroy()
