@@ -9,7 +9,7 @@
 //
 // Work split: a workgroup of four waves computes a 128 (rows of x) by 64*NTW
 // (rows of w) block of y.  The activations of one 128-column step are staged in
-// LDS (double buffered) and shared by the four waves; every wave dequantizes
+// LDS by LDS-direct loads (double buffered) and shared by the four waves; every wave dequantizes
 // the codes of its own NTW tiles of 16 weight rows straight into the B-operand
 // registers of the matrix instruction (the stream-tile layout hands each lane
 // exactly the eight consecutive columns the instruction wants), so each weight
@@ -59,11 +59,14 @@ __device__ __forceinline__ void meta_to_half(uint32_t word, half8 &scale, half8 
 template <int NTW, bool BF>
 __global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
 {
-    // activation stage: [buffer][column octet][row ^ octet] of 16-byte pieces; the
-    // XOR spreads the 16 octets a quarter-wave writes for one row over the banks
-    // and keeps the 16 rows a quarter-wave reads for one octet contiguous
-    __shared__ uint4 a_lds[2][16][kGemmBM];
+    // Activation stage: [buffer][row][slot] of 16-byte pieces, slot = octet ^ (row % 16).
+    // It is filled by LDS-direct loads (no registers): one wave instruction brings four
+    // rows x 256 contiguous bytes; the XOR keeps the 16 rows a quarter-wave later reads
+    // for one octet on different banks.
+    __shared__ uint4 a_lds[2][kGemmBM][16];
     constexpr int MI = kGemmBM / 16;  // 16-row fragments of x per workgroup
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    typedef const __attribute__((address_space(1))) void *global_ptr;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -75,20 +78,30 @@ __global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
     const uint32_t step_begin = split * p.steps_per_split;
     const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
 
-    // this thread's part of the activation stage: rows (t/16 + 16*i), octet t%16
-    const uint32_t a_row = threadIdx.x >> 4, a_oct = threadIdx.x & 15u;
-    auto fetch_a = [&](uint32_t step, uint4 (&regs)[MI]) {
-        const uint32_t k = step * kStepColumns + a_oct * 8u;
+    // this lane's pieces of the activation stage: rows 32*wave + 4*j + lane/16, slot lane%16.
+    // Rows beyond M re-read the last row and columns beyond K re-read the previous group
+    // (finite values against zero weights): both stay in bounds and never reach y.
+    const _Float16 *a_source[MI];
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            const uint32_t m = m0 + a_row + 16u * i;
-            regs[i] = (m < p.M && k < p.K) ? *(const uint4 *)(p.x + (size_t)m * p.K + k)
-                                           : make_uint4(0u, 0u, 0u, 0u);
+    for (int j = 0; j < MI; ++j) {
+        const uint32_t local = 32u * wave + 4u * j + kq;
+        uint32_t m = m0 + local;
+        m = m < p.M ? m : p.M - 1u;
+        a_source[j] = p.x + (size_t)m * p.K + 8u * (r ^ (local & 15u));
+    }
+    auto fetch_a = [&](uint32_t step, int buffer) {
+#pragma unroll
+        for (int j = 0; j < MI; ++j) {
+            // the octet is already in a_source; only the K tail needs care: when K is an odd
+            // multiple of 64 the upper half of the last step does not exist, and the lane
+            // reads the lower half again (64 columns back, still inside its row)
+            const uint32_t k = step * kStepColumns;
+            const uint32_t octet = r ^ ((32u * wave + 4u * j + kq) & 15u);
+            const _Float16 *source = a_source[j] + k;
+            if (k + 8u * octet >= p.K) source -= 64;
+            __builtin_amdgcn_global_load_lds((global_ptr)source,
+                                             (lds_ptr)&a_lds[buffer][32u * wave + 4u * j][0], 16, 0, 0);
         }
-    };
-    auto store_a = [&](int buffer, const uint4 (&regs)[MI]) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i) a_lds[buffer][a_oct][(a_row + 16u * i) ^ a_oct] = regs[i];
     };
     uint4 b_codes[NTW];
     uint2 b_meta[NTW];
@@ -110,23 +123,32 @@ __global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
         for (int t = 0; t < NTW; ++t) acc[i][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     const NibbleMasks masks = nibble_masks();
 
-    uint4 a_regs[MI];
     if (step_begin < step_end) {
-        fetch_a(step_begin, a_regs);
+        fetch_a(step_begin, 0);
         fetch_b(step_begin, b_codes, b_meta);
-        store_a(0, a_regs);
     }
     for (uint32_t step = step_begin; step < step_end; ++step) {
         const int buffer = (int)((step - step_begin) & 1u);
         const bool more = step + 1u < step_end;
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces of the stage have landed
+        __syncthreads();                     // everyone's have; the other buffer is free again
         uint4 next_codes[NTW];
         uint2 next_meta[NTW];
         if (more) {
-            fetch_a(step + 1u, a_regs);
+            fetch_a(step + 1u, buffer ^ 1);
             fetch_b(step + 1u, next_codes, next_meta);
         }
-        __syncthreads();  // stage `buffer` is complete; the other one is free again
 
+        // A fragments of the next half-quarter are read from LDS while the matrix
+        // instructions of this one run (two register sets, static indices).
+        constexpr int HALF = MI / 2;
+        half8 a_frag[2][HALF];
+        auto read_a = [&](int d, int h, half8 (&frags)[HALF]) {
+#pragma unroll
+            for (int i = 0; i < HALF; ++i)
+                frags[i] = __builtin_bit_cast(half8, a_lds[buffer][16 * (h * HALF + i) + r][(4 * d + kq) ^ r]);
+        };
+        read_a(0, 0, a_frag[0]);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             half8 b_frag[NTW];
@@ -139,16 +161,21 @@ __global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
                 b_frag[t] = dequant8(word, masks, scale, bias);
             }
 #pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                const half8 a_frag = __builtin_bit_cast(half8, a_lds[buffer][4 * d + kq][(16 * i + r) ^ (4 * d + kq)]);
+            for (int h = 0; h < 2; ++h) {
+                const int current = (2 * d + h) & 1;
+                if (h == 0)
+                    read_a(d, 1, a_frag[current ^ 1]);
+                else if (d < 3)
+                    read_a(d + 1, 0, a_frag[current ^ 1]);
 #pragma unroll
-                for (int t = 0; t < NTW; ++t)
-                    acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag, b_frag[t], acc[i][t],
-                                                                       0, 0, 0);
+                for (int i = 0; i < HALF; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t)
+                        acc[h * HALF + i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            a_frag[current][i], b_frag[t], acc[h * HALF + i][t], 0, 0, 0);
             }
         }
         if (more) {
-            store_a(buffer ^ 1, a_regs);
 #pragma unroll
             for (int t = 0; t < NTW; ++t) {
                 b_codes[t] = next_codes[t];
