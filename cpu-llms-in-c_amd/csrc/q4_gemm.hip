@@ -57,7 +57,7 @@ __device__ __forceinline__ void meta_to_half(uint32_t word, half8 &scale, half8 
 }
 
 template <int NTW, bool BF>
-__global__ void __launch_bounds__(256) q4_gemm_kernel(const GemmParams p)
+__global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
 {
     // Activation stage: [buffer][row][slot] of 16-byte pieces, slot = octet ^ (row % 16).
     // It is filled by LDS-direct loads (no registers): one wave instruction brings four
