@@ -96,3 +96,11 @@ def test_agrees_with_streaming_kernel_rows(engine, gpu):
 def test_dtypes_and_residual(engine, oracle, gpu, x_dtype, y_dtype):
     run_case(engine, oracle, gpu, 384, 512, 40, engine.META_F16_INTERLEAVED, getattr(engine, x_dtype),
              getattr(engine, y_dtype), residual=True)
+
+
+@pytest.mark.parametrize("forced", ["0,1", "1,2", "2,1", "3,1", "3,3", "4,1", "5,2"])
+def test_forced_decompositions(engine, oracle, gpu, forced, monkeypatch):
+    """Every kernel variant the host heuristic can pick (rows per block, tiles per wave, odd
+    tile on the last wave), with and without K splits."""
+    monkeypatch.setenv("MI355Q_Q4_GEMM", forced)
+    run_case(engine, oracle, gpu, 1104, 2176, 150, engine.META_BF16_PLANES, engine.F16, engine.F32)
