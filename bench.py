@@ -20,6 +20,15 @@ dispatch, measured in a second pass of the same steps).  `cpu_baseline` is the
 CPU oracle (a C restatement of the reference's scalar loop, row-parallel with
 OpenMP as the reference parallelises its GEMV) timed on this host on the same
 layer.
+
+Other workloads (never the default; each prints its own JSON line of the same
+shape): `--workload prefill --rows 512` times the gate, up and down GEMMs of the
+same layer at M rows against the fp16 matrix-instruction peak (2*M*K*N flops per
+linear); `--workload w8a8` times one activation quantization and the three
+projections that share it (M=64, K=1024, N=4096) in int8 with int32
+accumulators, and checks the accumulators bit for bit against the CPU oracle in
+the cpu_baseline leg; `--rows 2..8` turns the default workload into the
+small-M verify case.
 """
 from __future__ import annotations
 
@@ -37,6 +46,8 @@ sys.path.insert(0, str(ROOT / "cpu-llms-in-c_amd"))
 sys.path.insert(0, str(ROOT / "oracle"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X datasheet: 8 TB/s HBM3E
+F16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 matrix instructions
+I8_MFMA_PEAK_TOPS = 5000.0  # dense int8 matrix instructions
 
 LAYER = [  # name, N (output rows), K (input columns)
     ("q_proj", 6144, 5120),
@@ -48,6 +59,8 @@ LAYER = [  # name, N (output rows), K (input columns)
     ("down_proj", 5120, 17408),
 ]
 CONFIG1 = [("linear_0p8b", 3584, 1024)]
+PREFILL = [("gate_proj", 17408, 5120), ("up_proj", 17408, 5120), ("down_proj", 5120, 17408)]
+W8A8 = {"M": 64, "K": 1024, "N": 4096, "projections": 3}
 
 
 def q4_bytes(N, K, M, y_bytes=2):
@@ -111,6 +124,194 @@ def cpu_baseline(oracle, shapes, host, M, meta_kind, repeats=5):
                   f"cpu_row_dot, OpenMP static over rows, {median * 1e3:.1f} ms per pass",
     }
 
+def time_steps(ctx, run_steps, steps, warmup):
+    """Wall and event time of `steps` steps after `warmup`, then the same steps again with an
+    event pair around every dispatch: (wall s, gpu ms, sum of kernel ms, kernel launches)."""
+    run_steps(warmup)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_begin()
+    run_steps(steps)
+    gpu_ms = ctx.timer_end()  # waits for the stream
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    ctx.profile_begin()
+    run_steps(steps)
+    kernel_ms, launches = ctx.profile_end()
+    return wall, gpu_ms, kernel_ms, launches
+
+
+def common_fields(args, wall):
+    return {
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+    }
+
+
+def device_fields(info):
+    return {"device": info.name.decode(errors="replace").strip(),
+            "arch": info.arch.decode(errors="replace"), "compute_units": info.compute_units}
+
+
+def bench_prefill(engine, ctx, args):
+    """gate, up (one call, shared activations) and down at M rows: fp16 matrix-instruction GEMMs."""
+    M = args.rows
+    copies = 2
+    meta_kind = engine.META_BF16_PLANES
+    weights, host, x_ptr, y_ptr = [[] for _ in range(copies)], {}, {}, {}
+    for index, (name, N, K) in enumerate(PREFILL):
+        host[name] = engine.synth_q4_affine(1004 + index, 0.02, N, K, meta_kind)
+        for copy in range(copies):
+            weights[copy].append(ctx.q4_prepare(*host[name], N, K, meta_kind))
+        if K not in x_ptr:
+            host[("x", K)] = engine.synth_normal_f16(77 + K, 1.0, M * K).reshape(M, K)
+            x_ptr[K] = ctx.to_device(host[("x", K)])
+        y_ptr[name] = ctx.alloc(M * N * 2)
+    calls = []
+    for copy in range(copies):
+        gate, up, down = weights[copy]
+        calls.append(engine.make_calls([
+            ([(gate, y_ptr["gate_proj"]), (up, y_ptr["up_proj"])], x_ptr[5120], engine.F16, M, engine.F16),
+            ((down, y_ptr["down_proj"]), x_ptr[17408], engine.F16, M, engine.F16)]))
+
+    def run_steps(count):
+        for step in range(count):
+            ctx.q4_sequence(calls[step % copies])
+
+    wall, gpu_ms, kernel_ms, launches = time_steps(ctx, run_steps, args.steps, args.warmup)
+    step_flops = sum(2.0 * M * N * K for _, N, K in PREFILL)
+    value = step_flops * args.steps / wall / 1e12
+    achieved = step_flops * args.steps / (kernel_ms * 1e-3) / 1e12
+    result = {
+        "metric": "q4_prefill_tflops_m%d_27b_mlp" % M,
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        **common_fields(args, wall),
+        "dtype": "u4 codes dequantized to f16, f16 matrix instructions, f32 accumulate",
+        "data": "synthetic (seeded N(0,0.02) weights min/max-quantized to affine-Q4 g64, N(0,1) "
+                "fp16 activations)",
+        "config": {
+            "workload": "27B-shaped MLP linears gate/up (5120->17408) and down (17408->5120) at M=%d, "
+                        "affine-Q4 g64, bf16 scale+bias, fp16 x and y" % M,
+            "linears_per_step": 3,
+            "algorithmic_flops_per_step": step_flops,
+            "percent_of_f16_peak": round(100.0 * value / F16_MFMA_PEAK_TFLOPS, 2),
+            "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
+            **device_fields(ctx.info()),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": F16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / F16_MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "kernel": "q4_gemm_kernel (with its split-K reduction where one runs)",
+            "launches": int(launches),
+            "kernel_us_per_linear": round(kernel_ms * 1e3 / (3 * args.steps), 3),
+            "algorithmic_flops_per_linear": step_flops / 3,
+        },
+    }
+    if not args.no_cpu:
+        import oracle  # test infrastructure, used here only as the timed CPU baseline
+        threads = min(os.cpu_count() or 1, 16)
+        rows = min(M, 4)  # bounded sample: the first rows of the same activations
+        t0 = time.perf_counter()
+        for name, N, K in PREFILL:
+            oracle.q4_linear(*host[name], meta_kind, N, K, host[("x", K)][:rows], oracle.X_F16, rows,
+                             oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=threads)
+        seconds = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": round(step_flops * rows / M / seconds / 1e12, 5), "unit": "TFLOP/s",
+            "cores": threads, "kind": "port",
+            "sample": "the first %d of the %d rows through the three linears, oracle restatement of "
+                      "cpu_row_dot, OpenMP static over output rows, %.2f s" % (rows, M, seconds)}
+    print(json.dumps(result), flush=True)
+    for copy in weights:
+        for weight in copy:
+            weight.destroy()
+    return 0
+
+
+def bench_w8a8(engine, ctx, args):
+    """One step: quantize the activations once, then three projections that share them."""
+    M, K, N, count = W8A8["M"], W8A8["K"], W8A8["N"], W8A8["projections"]
+    rows = [engine.synth_w8_rows(2000 + i, 0.02, N, K) for i in range(count)]
+    weights = [ctx.w8a8_prepare(r, N, K) for r in rows]
+    x = engine.synth_normal_f32(31, 1.0, M * K).reshape(M, K)
+    bias = [engine.synth_normal_f32(41 + i, 0.1, N) for i in range(count)]
+    x_ptr, q_ptr, s_ptr = ctx.to_device(x), ctx.alloc(M * K), ctx.alloc(M * 4)
+    bias_ptr = [ctx.to_device(b) for b in bias]
+    out_ptr = [ctx.alloc(M * N * 4) for _ in range(count)]
+    acc_ptr = [ctx.alloc(M * N * 4) for _ in range(count)]
+
+    def run_steps(steps):
+        for _ in range(steps):
+            ctx.quantize_i8_device(x_ptr, M, K, q_ptr, s_ptr)
+            for i in range(count):
+                ctx.w8a8_linear_device(weights[i], q_ptr, s_ptr, M, bias_ptr[i], out_ptr[i], acc_ptr[i])
+
+    wall, gpu_ms, kernel_ms, launches = time_steps(ctx, run_steps, args.steps, args.warmup)
+    step_ops = 2.0 * M * K * N * count
+    value = step_ops * args.steps / wall / 1e12
+    achieved = step_ops * args.steps / (kernel_ms * 1e-3) / 1e12
+    result = {
+        "metric": "w8a8_tops_m64_k1024_n4096",
+        "value": round(value, 3),
+        "unit": "TOP/s",
+        **common_fields(args, wall),
+        "dtype": "i8 x i8, i32 accumulate, f32 epilogue",
+        "data": "synthetic (seeded N(0,0.02) weights absmax-quantized per row, N(0,1) fp32 activations "
+                "quantized per token on the GPU)",
+        "config": {
+            "workload": "per-token int8 quantization then %d projections M=%d K=%d N=%d with bias"
+                        % (count, M, K, N),
+            "launches_per_step": 1 + count,
+            "algorithmic_ops_per_step": step_ops,
+            "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
+            **device_fields(ctx.info()),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved, 3),
+            "peak": I8_MFMA_PEAK_TOPS,
+            "unit": "TOP/s",
+            "frac": round(achieved / I8_MFMA_PEAK_TOPS, 5),
+            "traffic": None,
+            "kernel": "w8a8_kernel (quantize_i8_kernel included in the time)",
+            "launches": int(launches),
+            "avg_kernel_us": round(kernel_ms * 1e3 / max(launches, 1), 3),
+        },
+    }
+    if not args.no_cpu:
+        import oracle  # test infrastructure: the timed CPU baseline and the bit-exactness check
+        threads = min(os.cpu_count() or 1, 16)
+        q_ref, s_ref = oracle.quantize_i8(x)
+        repeats, t0 = 20, time.perf_counter()
+        for _ in range(repeats):
+            oracle.quantize_i8(x)
+            refs = [oracle.w8a8_linear(rows[i], N, K, q_ref, s_ref, bias[i], threads=threads)
+                    for i in range(count)]
+        seconds = (time.perf_counter() - t0) / repeats
+        exact = bool(np.array_equal(ctx.download(q_ptr, (M, K), np.int8), q_ref))
+        for i in range(count):
+            exact &= bool(np.array_equal(ctx.download(acc_ptr[i], (M, N), np.int32), refs[i][1]))
+            exact &= bool(np.array_equal(ctx.download(out_ptr[i], (M, N), np.float32), refs[i][0]))
+        result["config"]["bit_exact_vs_oracle"] = exact
+        result["cpu_baseline"] = {
+            "value": round(step_ops / seconds / 1e12, 5), "unit": "TOP/s", "cores": threads, "kind": "port",
+            "sample": "%d passes of the same step (mean), oracle restatement of quantize_i8 and "
+                      "matrix_sequence_i8_quantized, OpenMP static over output rows, %.2f ms per pass" % (repeats, seconds * 1e3)}
+    print(json.dumps(result), flush=True)
+    for weight in weights:
+        ctx.w8a8_destroy(weight)
+    return 0
+
 
 def main():
     parser = argparse.ArgumentParser()
@@ -118,8 +319,9 @@ def main():
     parser.add_argument("--steps", type=int, default=400)
     parser.add_argument("--warmup", type=int, default=40)
     parser.add_argument("--copies", type=int, default=8)
-    parser.add_argument("--rows", type=int, default=1, help="activation rows M (1..8)")
-    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1"])
+    parser.add_argument("--rows", type=int, default=None,
+                        help="activation rows M (default 1; 512 for --workload prefill)")
+    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "prefill", "w8a8"])
     parser.add_argument("--unfused", action="store_true",
                         help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
     parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -132,6 +334,13 @@ def main():
 
     import mi355q as engine  # raises if the library is not built
 
+    if args.rows is None:
+        args.rows = 512 if args.workload == "prefill" else 1
+    if args.workload in ("prefill", "w8a8"):
+        if args.steps == 400 and args.warmup == 40:
+            args.steps, args.warmup = 100, 10
+        with engine.Context(0) as ctx:  # raises without a GPU
+            return (bench_prefill if args.workload == "prefill" else bench_w8a8)(engine, ctx, args)
     shapes = LAYER if args.workload == "layer_m1" else CONFIG1
     meta_kind = engine.META_BF16_PLANES if args.workload == "layer_m1" else engine.META_F16_INTERLEAVED
     M = args.rows
@@ -170,8 +379,8 @@ def main():
     avg_kernel_us = kernel_ms * 1e3 / max(launches, 1)
     achieved = bytes_per_launch / (avg_kernel_us * 1e-6) / 1e9
     result = {
-        "metric": "q4_gemv_hbm_gb_per_s_m1_27b_layer" if args.workload == "layer_m1"
-                  else "q4_gemv_hbm_gb_per_s_m1_k1024_n3584",
+        "metric": ("q4_gemv_hbm_gb_per_s_m%d_27b_layer" % M) if args.workload == "layer_m1"
+                  else "q4_gemv_hbm_gb_per_s_m%d_k1024_n3584" % M,
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,

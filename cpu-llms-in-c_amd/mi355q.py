@@ -282,6 +282,16 @@ class Context:
               _ptr(acc), 0)
         return out, acc
 
+    def quantize_i8_device(self, x_ptr: int, M: int, K: int, q_ptr: int, scales_ptr: int,
+                           asynchronous: bool = True):
+        _call(self.lib.mi355q_quantize_i8, self.handle, x_ptr, M, K, q_ptr, scales_ptr,
+              X_DEVICE | Y_DEVICE | (ASYNC if asynchronous else 0))
+
+    def w8a8_linear_device(self, weight, q_ptr: int, scales_ptr: int, M: int, bias_ptr, out_ptr: int,
+                           acc_ptr=None, asynchronous: bool = True):
+        _call(self.lib.mi355q_w8a8_linear, self.handle, weight, q_ptr, scales_ptr, M, bias_ptr, out_ptr,
+              acc_ptr, X_DEVICE | Y_DEVICE | (ASYNC if asynchronous else 0))
+
     def q4_sequence(self, calls):
         """calls: a ctypes array of Q4Call (build once, reuse)."""
         _call(self.lib.mi355q_q4_linear_sequence, self.handle, calls, len(calls))
