@@ -10,15 +10,23 @@
 // vector of ones; scale and bias are applied per group in fp32.  The weight is
 // never rounded.
 //
-// Work split: a workgroup owns TB tiles (16 output rows each) and keeps the
-// activations in LDS.  Its W waves take the 128-column steps round-robin (wave
-// w: steps w, w+W, ...); each wave keeps D steps of loads in flight.  Partial sums
-// meet in LDS and are added in wave order (a fixed order: results do not
-// depend on timing).  Nothing is shared between workgroups.  Long rows with
-// many activation rows are walked in column chunks so the activations fit LDS.
+// Work split: a workgroup owns TB tiles (16 output rows each).  Its W waves take
+// the 128-column steps round-robin (wave w: steps w, w+W, ...); each wave keeps D
+// steps of loads in flight.  Partial sums meet in LDS and are added in wave order
+// (a fixed order: results do not depend on timing).  Nothing is shared between
+// workgroups.
+//
+// The workgroup copies the activations of its columns into LDS (laid out
+// [octet of columns][row], so a wave's fragment reads are contiguous) and every
+// wave reads its steps from there.  With several activation rows that copy is as
+// large as the weights a tile brings, so a workgroup then takes two tiles, long
+// rows are cut in slices over workgroups (fp32 partial sums, added in slice order
+// by a second small kernel), and a slice that still overflows LDS is walked in
+// chunks.
 #include "device_util.h"
 #include "internal.h"
 
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -36,8 +44,13 @@ struct StreamParams {
     const _Float16 *x;  // [rows][K] fp16
     uint32_t M, K, T;
     uint32_t rows;         // M, or 2*M when fp32 activations are carried as (value, remainder) pairs
-    uint32_t chunks;       // column chunks (1 unless the activations overflow the LDS budget)
-    uint32_t chunk_steps;  // steps per chunk (the last chunk may be shorter, never shorter than W)
+    // The T steps are cut in `slices` runs of slice_steps (workgroups with blockIdx.y == s
+    // take run s); a workgroup walks its run in chunks of chunk_steps, the activations of
+    // one chunk in LDS at a time.  With more than one slice the workgroups write fp32
+    // partial sums [slice][M][n_total] for the reduction kernel.
+    uint32_t slices, slice_steps, chunk_steps;
+    float *partials;
+    uint32_t n_total, n_first[kMaxTargets];
     int pair;
     int y_dtype, residual_dtype;
     int meta_bf16;
@@ -88,10 +101,10 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const half8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
     const NibbleMasks masks = nibble_masks();
     const uint4 *xs_lane = xs + kq * MP + (r & (MP - 1));
-
-    for (uint32_t chunk = 0; chunk < p.chunks; ++chunk) {
-        const uint32_t first = chunk * p.chunk_steps;
-        const uint32_t last = first + p.chunk_steps < p.T ? first + p.chunk_steps : p.T;
+    const uint32_t slice_begin = blockIdx.y * p.slice_steps;
+    const uint32_t slice_end = slice_begin + p.slice_steps < p.T ? slice_begin + p.slice_steps : p.T;
+    for (uint32_t first = slice_begin; first < slice_end; first += p.chunk_steps) {
+        const uint32_t last = first + p.chunk_steps < slice_end ? first + p.chunk_steps : slice_end;
         // this wave's steps in the chunk: first + wave + i*W, i < count
         const uint32_t span = last - first;
         const uint32_t count = wave < span ? (span - wave + W - 1u) / W : 0u;
@@ -113,20 +126,22 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
         // The activation loads go out first (they come back from L2 quickly),
         // then the first D weight steps; the LDS stores wait for the former only.
-        constexpr int SB = 4;
+        constexpr int SB = MP == 1 ? 5 : 10;  // fetches in flight per thread: one L2 round trip for most slices
         const uint32_t octets = span * 16u;
         const uint32_t items = octets * MP;
         auto stage_fetch = [&](uint32_t index) {
             uint4 v = make_uint4(0u, 0u, 0u, 0u);
             if (index < items) {
-                const uint32_t mrow = index / octets, o = index % octets;
+                // consecutive threads fill consecutive LDS slots (no bank conflicts); each
+                // activation row still contributes runs of 64/MP adjacent octets
+                const uint32_t mrow = index % MP, o = index / MP;
                 const uint32_t k = first * kStepColumns + o * 8u;
                 if (mrow < p.rows && k < p.K) v = *(const uint4 *)(p.x + (size_t)mrow * p.K + k);
             }
             return v;
         };
         auto stage_store = [&](uint32_t index, const uint4 &v) {
-            if (index < items) xs[(size_t)(index % octets) * MP + index / octets] = v;
+            if (index < items) xs[index] = v;
         };
         uint4 staged[SB];
 #pragma unroll
@@ -136,7 +151,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 #pragma unroll
         for (int u = 0; u < D; ++u) issue(u, ring[u]);
 
-        if (chunk > 0) __syncthreads();  // everyone is done with the previous chunk
+        if (first > slice_begin) __syncthreads();  // everyone is done with the previous chunk
 #pragma unroll
         for (int b = 0; b < SB; ++b) stage_store(threadIdx.x + b * 64u * W, staged[b]);
         for (uint32_t base = threadIdx.x + SB * 64u * W; base < items; base += SB * 64u * W) {
@@ -221,11 +236,34 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 value += v[(j + 1) % NJ];
                 m = row >> 1;
             }
+            if (p.slices > 1u) {
+                p.partials[((size_t)blockIdx.y * p.M + m) * p.n_total + p.n_first[target] + n] = value;
+                continue;
+            }
             const size_t at = (size_t)m * N + n;
             if (p.residual[target]) value += load_as_float(p.residual[target], p.residual_dtype, at);
             store_from_float(p.y[target], p.y_dtype, at, value);
         }
     }
+}
+
+// Adds the slices' partial sums in slice order (a fixed order) and applies the
+// epilogue.  One thread per output element of all targets.
+__global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParams p)
+{
+    const uint32_t column = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t m = blockIdx.y;
+    if (column >= p.n_total) return;
+    uint32_t target = 0;
+#pragma unroll
+    for (uint32_t t = 1; t < kMaxTargets; ++t)
+        if (t < p.targets && column >= p.n_first[t]) target = t;
+    float value = 0.0f;
+    for (uint32_t s = 0; s < p.slices; ++s)
+        value += p.partials[((size_t)s * p.M + m) * p.n_total + column];
+    const size_t at = (size_t)m * p.N[target] + (column - p.n_first[target]);
+    if (p.residual[target]) value += load_as_float(p.residual[target], p.residual_dtype, at);
+    store_from_float(p.y[target], p.y_dtype, at, value);
 }
 
 // Activations that are not fp16 are converted once per call into fp16 rows:
@@ -254,24 +292,29 @@ q4_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__restric
 
 struct StreamShape {
     int mp, tb, depth, waves;
-    uint32_t chunks, chunk_steps;
+    uint32_t slices, slice_steps, chunk_steps;
 };
+
+static size_t stream_lds_bytes(int mp, int tb, int waves, uint32_t chunk_steps)
+{
+    const int nj = mp < 4 ? mp : 4;
+    return (size_t)chunk_steps * 256u * mp + (size_t)waves * tb * nj * 256u;
+}
 
 template <int MP, int TB, int D, int W>
 static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
 {
-    constexpr int NJ = MP < 4 ? MP : 4;
     uint32_t blocks = 0;
     for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
-    const size_t lds = (size_t)p.chunk_steps * 16u * MP * sizeof(uint4) +
-                       (size_t)W * TB * NJ * 64u * sizeof(float);
+    const size_t lds = stream_lds_bytes(MP, TB, W, p.chunk_steps);
+    const dim3 grid(blocks, p.slices);
     if (p.meta_bf16)
-        return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, dim3(blocks), dim3(64u * W), lds, p);
-    return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, dim3(blocks), dim3(64u * W), lds, p);
+        return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, grid, dim3(64u * W), lds, p);
+    return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, grid, dim3(64u * W), lds, p);
 }
 
 template <int MP>
-static hipError_t launch_mp(mi355q_context *ctx, const StreamParams &p, const StreamShape &shape)
+static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const StreamShape &shape)
 {
     switch (shape.tb * 10000 + shape.depth * 100 + shape.waves) {
     case 10202: return launch_one<MP, 1, 2, 2>(ctx, p);
@@ -279,34 +322,26 @@ static hipError_t launch_mp(mi355q_context *ctx, const StreamParams &p, const St
     case 10208: return launch_one<MP, 1, 2, 8>(ctx, p);
     case 10404: return launch_one<MP, 1, 4, 4>(ctx, p);
     case 10408: return launch_one<MP, 1, 4, 8>(ctx, p);
+    case 20202: return launch_one<MP, 2, 2, 2>(ctx, p);
     case 20204: return launch_one<MP, 2, 2, 4>(ctx, p);
     case 20208: return launch_one<MP, 2, 2, 8>(ctx, p);
+    case 40202: return launch_one<MP, 4, 2, 2>(ctx, p);
+    case 40204: return launch_one<MP, 4, 2, 4>(ctx, p);
+    case 40208: return launch_one<MP, 4, 2, 8>(ctx, p);
     default: return hipErrorInvalidValue;
     }
 }
 
-static size_t stream_lds_bytes(int mp, int tb, int waves, uint32_t chunk_steps)
-{
-    return (size_t)chunk_steps * 256u * mp + (size_t)waves * tb * 1024u;
-}
-
-// Column chunks: the activation slice may take up to 40 KiB of LDS, and even
-// the last chunk must give every wave a step.
-static void choose_chunks(StreamShape &shape, uint32_t T)
+// Cuts the T steps into slices (across workgroups) and each slice into chunks
+// (walked by one workgroup) whose activations take at most 40 KiB of LDS.
+static void choose_cuts(StreamShape &shape, uint32_t T, uint32_t slices)
 {
     const uint32_t max_steps = (40u * 1024u) / (256u * (uint32_t)shape.mp);
-    uint32_t chunks = (T + max_steps - 1) / max_steps;
-    uint32_t each = T;
-    for (; chunks > 1u; --chunks) {
-        each = (T + chunks - 1) / chunks;
-        if ((chunks - 1u) * each < T && T - (chunks - 1u) * each >= (uint32_t)shape.waves) break;
-    }
-    if (chunks <= 1u) {
-        chunks = 1u;
-        each = T;
-    }
-    shape.chunks = chunks;
-    shape.chunk_steps = each;
+    slices = slices < 1u ? 1u : slices > T ? T : slices;
+    shape.slice_steps = (T + slices - 1) / slices;
+    shape.slices = (T + shape.slice_steps - 1) / shape.slice_steps;
+    const uint32_t chunks = (shape.slice_steps + max_steps - 1) / max_steps;
+    shape.chunk_steps = (shape.slice_steps + chunks - 1) / chunks;
 }
 
 static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp)
@@ -314,30 +349,39 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
     StreamShape shape;
     shape.mp = mp;
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
-    // about 4-5 thousand waves with two steps of loads in flight each keeps HBM
-    // busy without queueing; more waves per workgroup when there are few tiles
     shape.tb = 1;
     shape.depth = 2;
-    const uint32_t want = (16u * cus + NT_total - 1) / NT_total;
-    shape.waves = want <= 2u ? 2 : want <= 5u ? 4 : 8;
-    while (shape.waves > 2 && (uint32_t)shape.waves > T) shape.waves /= 2;
-    const char *force = getenv("MI355Q_Q4_STREAM");  // "TB,DEPTH,WAVES" for experiments
-    int ft = 0, fd = 0, fw = 0;
-    if (force && sscanf(force, "%d,%d,%d", &ft, &fd, &fw) == 3) {
+    uint32_t slices = 1;
+    if (mp == 1) {
+        // about 4-5 thousand waves with two steps of loads in flight each keeps HBM
+        // busy without queueing; more waves per workgroup when there are few tiles
+        const uint32_t want = (16u * cus + NT_total - 1) / NT_total;
+        shape.waves = want <= 2u ? 2 : want <= 5u ? 4 : 8;
+    } else {
+        // every workgroup copies its activation rows from L2 into LDS: two tiles per
+        // workgroup halve that traffic.  Matrices with few tiles and long rows are cut in
+        // slices (of 32 steps or more: the reduction launch costs about as much as
+        // 10 steps) until some 2.5 workgroups per compute unit exist.
+        shape.tb = NT_total >= cus ? 2 : 1;
+        const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
+        slices = (5u * cus / 2u + groups / 2u) / groups;
+        if (slices > T / 32u) slices = T / 32u;
+        choose_cuts(shape, T, slices);
+        const uint32_t want = (16u * cus + groups * shape.slices - 1) / (groups * shape.slices);
+        shape.waves = want <= 2u ? 2 : want <= 8u ? 4 : 8;
+    }
+    // "TB,DEPTH,WAVES[,SLICES]" for experiments
+    const char *force = getenv("MI355Q_Q4_STREAM");
+    int ft = 0, fd = 0, fw = 0, fs = 0;
+    const int fields = force ? sscanf(force, "%d,%d,%d,%d", &ft, &fd, &fw, &fs) : 0;
+    if (fields >= 3) {
         shape.tb = ft;
         shape.depth = fd;
         shape.waves = fw;
+        if (fields >= 4 && fs >= 1) slices = (uint32_t)fs;
     }
-    choose_chunks(shape, T);
-    // fall back to smaller workgroups when the activations crowd LDS
-    if (stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps) > 64u * 1024u) {
-        shape.waves = 4;
-        choose_chunks(shape, T);
-    }
-    if (stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps) > 64u * 1024u) {
-        shape.tb = 1;
-        choose_chunks(shape, T);
-    }
+    choose_cuts(shape, T, mp == 1 ? 1u : slices);
+    while (shape.waves > 2 && (uint32_t)shape.waves > shape.chunk_steps) shape.waves /= 2;
     return shape;
 }
 
@@ -388,8 +432,19 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.K = first.K;
     p.T = first.T;
     p.rows = rows;
-    p.chunks = shape.chunks;
     p.chunk_steps = shape.chunk_steps;
+    p.slice_steps = shape.slice_steps;
+    p.slices = shape.slices;
+    if (p.slices > 1u) {
+        for (uint32_t t = 0; t < a.count; ++t) {
+            p.n_first[t] = p.n_total;
+            p.n_total += a.targets[t].w->N;
+        }
+        int status = ensure_stage(ctx, 4, (size_t)p.slices * a.M * p.n_total * sizeof(float), error,
+                                  error_capacity);
+        if (status != MI355Q_OK) return status;
+        p.partials = (float *)ctx->stage[4];
+    }
     p.pair = pair;
     p.y_dtype = a.y_dtype;
     p.residual_dtype = a.residual_dtype;
@@ -401,16 +456,27 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
                   lds, first.K, rows);
         return MI355Q_ERROR_INVALID;
     }
+    static const bool trace = getenv("MI355Q_TRACE") != nullptr;
+    if (trace)
+        fprintf(stderr, "mi355q: q4 stream rows=%u tiles=%u steps=%u -> %d tiles x %d waves per workgroup, "
+                        "depth %d, %u slices of %u steps in chunks of %u\n", rows, tiles, first.T, shape.tb,
+                shape.waves, shape.depth, shape.slices,
+                shape.slice_steps, shape.chunk_steps);
     hipError_t launched;
     switch (mp) {
-    case 1: launched = launch_mp<1>(ctx, p, shape); break;
-    case 2: launched = launch_mp<2>(ctx, p, shape); break;
-    case 4: launched = launch_mp<4>(ctx, p, shape); break;
-    case 8: launched = launch_mp<8>(ctx, p, shape); break;
-    default: launched = launch_mp<16>(ctx, p, shape); break;
+    case 1: launched = launch_shape<1>(ctx, p, shape); break;
+    case 2: launched = launch_shape<2>(ctx, p, shape); break;
+    case 4: launched = launch_shape<4>(ctx, p, shape); break;
+    case 8: launched = launch_shape<8>(ctx, p, shape); break;
+    default: launched = launch_shape<16>(ctx, p, shape); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 stream kernel launch", error, error_capacity);
+    if (p.slices > 1u) {
+        launched = launch(ctx, q4_stream_reduce_kernel, dim3((p.n_total + 255u) / 256u, a.M), dim3(256), 0, p);
+        if (launched != hipSuccess)
+            return fail_hip(launched, "q4 stream reduce launch", error, error_capacity);
+    }
     return MI355Q_OK;
 }
 

@@ -123,7 +123,9 @@ def test_argument_errors(engine, gpu):
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_shared_activation_multi_launch(engine, oracle, gpu, M):
     """q|k|v-style call: three weights of different row counts, one launch, same x; each output
-    must equal the single-weight call bit for bit and pass the oracle gate."""
+    must pass the oracle gate, repeat bit for bit on a second call, and agree with the
+    single-weight call to fp32 summation-order noise (the split of the columns over waves
+    depends on how many tiles a launch carries, so the order of the partial sums may differ)."""
     K = 1536
     rows = [640, 100, 1024]
     images = [engine.synth_q4_affine(60 + i, 0.02, N, K, engine.META_BF16_PLANES)
@@ -136,9 +138,12 @@ def test_shared_activation_multi_launch(engine, oracle, gpu, M):
         together = gpu.q4_linear_multi(weights, x, engine.F16, engine.F32)
         for (q, a, b), N, w, y in zip(images, rows, weights, together):
             alone = gpu.q4_linear(w, x, engine.F16, engine.F32)
-            assert np.array_equal(alone.view(np.uint32), y.view(np.uint32))
+            assert q4_relative_error(alone, y.astype(np.float64)) <= 1e-4
             ref = oracle.q4_linear(q, a, b, engine.META_BF16_PLANES, N, K, x, engine.F16, M)
             assert q4_relative_error(y, ref) <= TOLERANCE
+        again = gpu.q4_linear_multi(weights, x, engine.F16, engine.F32)
+        for first, second in zip(together, again):
+            assert np.array_equal(first.view(np.uint32), second.view(np.uint32))
         mixed = gpu.q4_prepare(*engine.synth_q4_affine(1, 0.02, 32, 512, engine.META_BF16_PLANES),
                                32, 512, engine.META_BF16_PLANES)
         with pytest.raises(engine.Mi355qError) as info:
