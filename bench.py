@@ -46,6 +46,10 @@ sys.path.insert(0, str(ROOT / "cpu-llms-in-c_amd"))
 sys.path.insert(0, str(ROOT / "oracle"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X datasheet: 8 TB/s HBM3E
+# HBM bytes moved per algorithmic byte by the streaming kernel on the default workload: FETCH_SIZE and
+# WRITE_SIZE of rocprofv3 --pmc, scaled by a plain 2 GiB read/fill in the same runs
+# (profiles/q4_stream_kernel_layer_m1.md); a counter reading, not something this script can measure
+MEASURED_TRAFFIC_RATIO_LAYER_M1 = 1.016
 F16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 matrix instructions
 I8_MFMA_PEAK_TOPS = 5000.0  # dense int8 matrix instructions
 
@@ -416,7 +420,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": round(bytes_per_launch * MEASURED_TRAFFIC_RATIO_LAYER_M1)
+                       if args.workload == "layer_m1" and M == 1 and not args.unfused else None,
             "kernel": "q4_stream_kernel",
             "launches": int(launches),
             "avg_kernel_us": round(avg_kernel_us, 3),
