@@ -359,6 +359,59 @@ void mi355q_q4_weight_destroy(mi355q_q4_weight *weight)
     delete weight;
 }
 
+int mi355q_sym128_weight_prepare(mi355q_context *ctx, const void *records, uint32_t N, uint32_t K,
+                                 int record_order, uint32_t flags, mi355q_q4_weight **out,
+                                 char *error, size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    if (ctx == nullptr || out == nullptr || records == nullptr) {
+        set_error(error, error_capacity, "sym128_weight_prepare: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (record_order != MI355Q_SYM128_ROW_MAJOR && record_order != MI355Q_SYM128_OUTPUT_BLOCKED) {
+        set_error(error, error_capacity, "sym128_weight_prepare: unknown record order %d", record_order);
+        return MI355Q_ERROR_INVALID;
+    }
+    if (N == 0 || K == 0 || K % 128u != 0 ||
+        (record_order == MI355Q_SYM128_OUTPUT_BLOCKED && N % 4u != 0)) {
+        set_error(error, error_capacity,
+                  "sym128_weight_prepare: shape %u x %u (columns must be a non-zero multiple of 128, "
+                  "rows of an output-blocked tensor a multiple of 4)", N, K);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t record_bytes = (size_t)N * (K / 128u) * 66u;
+    const size_t code_bytes = (size_t)N * (K / 2u), plane_bytes = (size_t)N * (K / 64u) * 2u;
+    // records (when they come from the host) | codes | scales | biases, each 256-byte aligned
+    const size_t at_codes = (flags & MI355Q_SOURCE_DEVICE) ? 0 : (record_bytes + 255u) & ~(size_t)255u;
+    const size_t at_scales = at_codes + ((code_bytes + 255u) & ~(size_t)255u);
+    const size_t at_biases = at_scales + ((plane_bytes + 255u) & ~(size_t)255u);
+    char *scratch = nullptr;
+    MI355Q_HIP(hipMalloc((void **)&scratch, at_biases + plane_bytes), "sym128 conversion buffer");
+    const uint8_t *source = (const uint8_t *)records;
+    hipError_t status = hipSuccess;
+    if (!(flags & MI355Q_SOURCE_DEVICE)) {
+        status = hipMemcpyAsync(scratch, records, record_bytes, hipMemcpyHostToDevice, ctx->stream);
+        source = (const uint8_t *)scratch;
+    }
+    if (status == hipSuccess)
+        status = sym128_to_affine_launch(source, record_order == MI355Q_SYM128_OUTPUT_BLOCKED, N, K,
+                                         (uint8_t *)(scratch + at_codes),
+                                         (uint16_t *)(scratch + at_scales),
+                                         (uint16_t *)(scratch + at_biases), ctx->stream);
+    int code = MI355Q_OK;
+    if (status != hipSuccess)
+        code = fail_hip(status, "sym128 conversion", error, error_capacity);
+    else  // stream order: the re-tiling kernels run after the conversion
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_codes, scratch + at_scales, scratch + at_biases,
+                                        N, K, MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, out, error,
+                                        error_capacity);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(scratch);
+    if (code == MI355Q_OK) (*out)->image_bytes = record_bytes;
+    return code;
+}
+
 size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight)
 {
     return weight ? weight->image_bytes : 0;
@@ -400,6 +453,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
     }
     const bool x_dev = flags & MI355Q_X_DEVICE, y_dev = flags & MI355Q_Y_DEVICE;
     const bool r_dev = !any_residual || (flags & MI355Q_RESIDUAL_DEVICE);
+    const bool is_bias = (flags & MI355Q_RESIDUAL_IS_BIAS) != 0;
     if ((flags & MI355Q_ASYNC) && !(x_dev && y_dev && r_dev)) {
         set_error(error, error_capacity, "q4_linear: ASYNC needs device pointers throughout");
         return MI355Q_ERROR_INVALID;
@@ -418,7 +472,9 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
         y_offset[t] = y_total;
         y_total += (cells * dtype_bytes(y_dtype) + 255u) & ~(size_t)255u;
         r_offset[t] = r_total;
-        if (targets[t].residual) r_total += (cells * dtype_bytes(residual_dtype) + 255u) & ~(size_t)255u;
+        const size_t r_cells = is_bias ? targets[t].weight->dev.N : cells;
+        if (targets[t].residual)
+            r_total += (r_cells * dtype_bytes(residual_dtype) + 255u) & ~(size_t)255u;
     }
 
     Q4LinearArgs args;
@@ -428,6 +484,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
     args.M = M;
     args.y_dtype = y_dtype;
     args.residual_dtype = residual_dtype;
+    args.residual_is_bias = is_bias;
     args.count = count;
     int status;
     if (!x_dev) {
@@ -447,7 +504,8 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
         args.targets[t].residual = targets[t].residual;
         if (targets[t].residual && !r_dev) {
             void *staged = (char *)ctx->stage[2] + r_offset[t];
-            MI355Q_HIP(hipMemcpyAsync(staged, targets[t].residual, cells * dtype_bytes(residual_dtype),
+            const size_t r_cells = is_bias ? targets[t].weight->dev.N : cells;
+            MI355Q_HIP(hipMemcpyAsync(staged, targets[t].residual, r_cells * dtype_bytes(residual_dtype),
                                       hipMemcpyHostToDevice, ctx->stream),
                        "residual upload");
             args.targets[t].residual = staged;

@@ -115,6 +115,10 @@ inline bool dtype_valid(int dtype) {
 hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
                             const uint16_t *meta_b, const Q4Device &dst,
                             hipStream_t stream);
+// symmetric group-128 records -> affine group-64 planes (all device pointers)
+hipError_t sym128_to_affine_launch(const uint8_t *records, int output_blocked, uint32_t N,
+                                   uint32_t K, uint8_t *quants, uint16_t *scales,
+                                   uint16_t *biases, hipStream_t stream);
 
 // q4_stream.hip
 constexpr uint32_t kMaxTargets = 4;
@@ -130,6 +134,7 @@ struct Q4LinearArgs {
     uint32_t M;
     int y_dtype;
     int residual_dtype;
+    bool residual_is_bias;  // residual is one row [N] added to every activation row
     uint32_t count;
     Q4Target targets[kMaxTargets];
 };

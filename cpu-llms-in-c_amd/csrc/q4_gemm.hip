@@ -38,6 +38,7 @@ struct GemmParams {
     uint32_t tiles_per_block;
     uint32_t splits, steps_per_split;
     int y_dtype, residual_dtype;
+    int residual_is_bias;  // residual is one row [N], added to every activation row
 };
 
 __device__ __forceinline__ half8 dequant8(uint32_t word, const NibbleMasks &masks, half8 scale,
@@ -233,7 +234,8 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
                     p.partials[(size_t)split * p.M * p.N + at] = acc[i][t][j];
                 } else {
                     float value = acc[i][t][j];
-                    if (p.residual) value += load_as_float(p.residual, p.residual_dtype, at);
+                    if (p.residual)
+                        value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? n : at);
                     store_from_float(p.y, p.y_dtype, at, value);
                 }
             }
@@ -248,7 +250,8 @@ __global__ void __launch_bounds__(256) q4_gemm_reduce_kernel(const GemmParams p)
     if (at >= total) return;
     float value = 0.0f;
     for (uint32_t s = 0; s < p.splits; ++s) value += p.partials[(size_t)s * total + at];
-    if (p.residual) value += load_as_float(p.residual, p.residual_dtype, at);
+    if (p.residual)
+        value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? at % p.N : at);
     store_from_float(p.y, p.y_dtype, at, value);
 }
 
@@ -292,6 +295,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     p.T = w.T;
     p.y_dtype = a.y_dtype;
     p.residual_dtype = a.residual_dtype;
+    p.residual_is_bias = a.residual_is_bias;
 
     // Decomposition: BM rows x (4*NTW + EXTRA) tiles per workgroup, K split in `splits`.
     // The choice minimises a microsecond estimate fitted to sweeps over every variant

@@ -76,6 +76,49 @@ q4_repack_meta_kernel(const uint16_t *__restrict__ meta_a,
     dst[index] = make_uint2(out[0], out[1]);
 }
 
+// Symmetric group-128 records (bf16 scale + 64 code bytes, two's complement
+// nibbles; compiler/q4_image.py:120-146, qwen35_task.c:286-303) to affine group-64
+// planes: q = v + 8 (flip the nibble's top bit), scale unchanged, bias = -8 * scale
+// (a power-of-two multiple: exact in bf16).  One thread per 64-column group and
+// code word.
+__global__ void __launch_bounds__(256)
+sym128_to_affine_kernel(const uint8_t *__restrict__ records, int output_blocked, uint32_t N,
+                        uint32_t K, uint32_t *__restrict__ quants, uint16_t *__restrict__ scales,
+                        uint16_t *__restrict__ biases)
+{
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t groups = K / 128u;
+    const uint64_t total = (uint64_t)N * groups * 16u;  // 16 code words per record
+    if (index >= total) return;
+    const uint32_t word = (uint32_t)(index % 16u);
+    const uint64_t pair = index / 16u;  // (row, group)
+    const uint32_t row = (uint32_t)(pair / groups), g = (uint32_t)(pair % groups);
+    const uint64_t record_index =
+        output_blocked ? ((uint64_t)(row / 4u) * groups + g) * 4u + row % 4u : pair;
+    const uint8_t *record = records + record_index * 66u;
+    // records are only 2-byte aligned: assemble the word from bytes
+    const uint8_t *bytes = record + 2u + 4u * word;
+    const uint32_t codes = (uint32_t)bytes[0] | (uint32_t)bytes[1] << 8 | (uint32_t)bytes[2] << 16 |
+                           (uint32_t)bytes[3] << 24;
+    quants[pair * 16u + word] = codes ^ 0x88888888u;
+    if (word < 2u) {  // the two 64-column groups of this record
+        const uint16_t scale_bits = (uint16_t)(record[0] | record[1] << 8);
+        const float bias = -8.0f * __builtin_bit_cast(float, (uint32_t)scale_bits << 16);
+        scales[pair * 2u + word] = scale_bits;
+        biases[pair * 2u + word] = (uint16_t)(__builtin_bit_cast(uint32_t, bias) >> 16);
+    }
+}
+
+hipError_t sym128_to_affine_launch(const uint8_t *records, int output_blocked, uint32_t N,
+                                   uint32_t K, uint8_t *quants, uint16_t *scales,
+                                   uint16_t *biases, hipStream_t stream)
+{
+    const uint64_t total = (uint64_t)N * (K / 128u) * 16u;
+    hipLaunchKernelGGL(sym128_to_affine_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0,
+                       stream, records, output_blocked, N, K, (uint32_t *)quants, scales, biases);
+    return hipGetLastError();
+}
+
 hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
                             const uint16_t *meta_b, const Q4Device &dst,
                             hipStream_t stream)

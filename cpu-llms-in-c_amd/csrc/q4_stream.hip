@@ -53,6 +53,7 @@ struct StreamParams {
     uint32_t n_total, n_first[kMaxTargets];
     int pair;
     int y_dtype, residual_dtype;
+    int residual_is_bias;  // residual is one row [N], added to every activation row
     int meta_bf16;
 };
 
@@ -241,7 +242,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 continue;
             }
             const size_t at = (size_t)m * N + n;
-            if (p.residual[target]) value += load_as_float(p.residual[target], p.residual_dtype, at);
+            if (p.residual[target])
+                value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
             store_from_float(p.y[target], p.y_dtype, at, value);
         }
     }
@@ -261,8 +263,10 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
     float value = 0.0f;
     for (uint32_t s = 0; s < p.slices; ++s)
         value += p.partials[((size_t)s * p.M + m) * p.n_total + column];
-    const size_t at = (size_t)m * p.N[target] + (column - p.n_first[target]);
-    if (p.residual[target]) value += load_as_float(p.residual[target], p.residual_dtype, at);
+    const uint32_t n = column - p.n_first[target];
+    const size_t at = (size_t)m * p.N[target] + n;
+    if (p.residual[target])
+        value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
     store_from_float(p.y[target], p.y_dtype, at, value);
 }
 
@@ -448,6 +452,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.pair = pair;
     p.y_dtype = a.y_dtype;
     p.residual_dtype = a.residual_dtype;
+    p.residual_is_bias = a.residual_is_bias;
     p.meta_bf16 = first.meta_kind == MI355Q_META_BF16_PLANES;
 
     const size_t lds = stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps);

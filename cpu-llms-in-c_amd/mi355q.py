@@ -19,7 +19,8 @@ LIBRARY_PATH = PACKAGE_DIR / "lib" / "libmi355q.so"
 OK, ERROR_RUNTIME, ERROR_INVALID = 0, 1, 2
 F16, F32, BF16 = 0, 1, 2
 META_F16_INTERLEAVED, META_BF16_PLANES = 0, 1
-X_DEVICE, Y_DEVICE, RESIDUAL_DEVICE, ASYNC, SOURCE_DEVICE = 1, 2, 4, 8, 16
+X_DEVICE, Y_DEVICE, RESIDUAL_DEVICE, ASYNC, SOURCE_DEVICE, RESIDUAL_IS_BIAS = 1, 2, 4, 8, 16, 32
+SYM128_ROW_MAJOR, SYM128_OUTPUT_BLOCKED = 0, 1
 
 _c = ctypes
 _u32, _u64, _sz, _int = _c.c_uint32, _c.c_uint64, _c.c_size_t, _c.c_int
@@ -67,12 +68,17 @@ SIGNATURES = {
     "mi355q_probe_read_bandwidth": (_int, [_vp, _sz, _sz, _int, _int, _c.POINTER(_c.c_double), *_err]),
     "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
                                         _c.POINTER(_vp), *_err]),
+    "mi355q_sym128_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _int, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_multi": (_int, [_vp, _c.POINTER(Q4Target), _u32, _vp, _int, _u32, _int, _int,
                                       _u32, *_err]),
     "mi355q_q4_linear_sequence": (_int, [_vp, _c.POINTER(Q4Call), _sz, *_err]),
+    "mi355q_hook_q4_gemm": (_int, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
+    "mi355q_hook_q4_gemv": (_int, [_vp, _int, _sz, _sz, _vp, _vp]),
+    "mi355q_hook_last_error": (_int, [_c.c_char_p, _sz]),
+    "mi355q_hook_release": (None, []),
     "mi355q_w8a8_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_w8a8_weight_destroy": (None, [_vp]),
     "mi355q_quantize_i8": (_int, [_vp, _vp, _u32, _u32, _vp, _vp, _u32, *_err]),
@@ -226,14 +232,23 @@ class Context:
               _ptr(meta_b), N, K, meta_kind, flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
 
+    def sym128_prepare(self, records, N: int, K: int, record_order: int = SYM128_ROW_MAJOR,
+                       flags: int = 0) -> Q4Weight:
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_sym128_weight_prepare, self.handle, _ptr(records), N, K, record_order,
+              flags, ctypes.byref(out))
+        return Q4Weight(self, out, N, K)
+
     def q4_linear(self, weight: Q4Weight, x: np.ndarray, x_dtype: int, y_dtype: int = F32,
-                  residual: np.ndarray | None = None, residual_dtype: int = F32) -> np.ndarray:
+                  residual: np.ndarray | None = None, residual_dtype: int = F32,
+                  residual_is_bias: bool = False) -> np.ndarray:
         """Host-array convenience form: x [M][K] -> y [M][N]."""
         x = np.ascontiguousarray(x)
         M = x.shape[0]
         y = np.empty((M, weight.N), dtype=_NP_DTYPE[y_dtype])
         _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, _ptr(x), x_dtype, M,
-              _ptr(y), y_dtype, _ptr(residual), residual_dtype, 0)
+              _ptr(y), y_dtype, _ptr(residual), residual_dtype,
+              RESIDUAL_IS_BIAS if residual_is_bias else 0)
         return y
 
     def q4_linear_multi(self, weights, x: np.ndarray, x_dtype: int, y_dtype: int = F32):
@@ -315,6 +330,35 @@ def make_calls(items):
             slot.targets[index].y = target[1]
             slot.targets[index].residual = target[2] if len(target) > 2 else None
     return array
+
+
+# ---- entry points with the reference's hook signatures ----------------------
+
+def _hook_check(status: int):
+    if status != 0:
+        message = ctypes.create_string_buffer(256)
+        library().mi355q_hook_last_error(message, len(message))
+        raise Mi355qError(status, message.value.decode(errors="replace"))
+
+
+def hook_q4_gemm(records: np.ndarray, x: np.ndarray, N: int, bias=None) -> np.ndarray:
+    """output[r][n] = bias[n] + sum_k w[n][k] x[r][k]; records stay alive with the caller."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, K = x.shape
+    out = np.empty((rows, N), dtype=np.float32)
+    _hook_check(library().mi355q_hook_q4_gemm(_ptr(records), _ptr(x), rows, K, N, _ptr(bias), _ptr(out)))
+    return out
+
+
+def hook_q4_gemv(records: np.ndarray, record_order: int, N: int, x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(N, dtype=np.float32)
+    _hook_check(library().mi355q_hook_q4_gemv(_ptr(records), record_order, N, x.size, _ptr(x), _ptr(out)))
+    return out
+
+
+def hook_release():
+    library().mi355q_hook_release()
 
 
 # ---- synthetic inputs (host side) ------------------------------------------

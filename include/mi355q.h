@@ -64,7 +64,20 @@ enum {
     MI355Q_Y_DEVICE = 1u << 1,        /* y is a device pointer */
     MI355Q_RESIDUAL_DEVICE = 1u << 2, /* residual is a device pointer */
     MI355Q_ASYNC = 1u << 3,           /* do not wait; all pointers must be device */
-    MI355Q_SOURCE_DEVICE = 1u << 4    /* prepare: image pointers are device pointers */
+    MI355Q_SOURCE_DEVICE = 1u << 4,   /* prepare: image pointers are device pointers */
+    /* the residual is one row [N] added to every activation row: the `bias` of the
+     * reference's grouped linear (whisper_turbo_encoder.c:127-157) */
+    MI355Q_RESIDUAL_IS_BIAS = 1u << 5
+};
+
+/* record order of a symmetric group-128 Q4 tensor */
+enum {
+    /* record (n, g) at index n*(K/128) + g (compiler/q4_image.py:120-146) */
+    MI355Q_SYM128_ROW_MAJOR = 0,
+    /* four output rows interleaved: index ((n/4)*(K/128) + g)*4 + n%4
+     * (compiler/q4_image.py:44-61; KIND_Q4_OUTPUT_BLOCKED, qwen35_task.c:324-345,432-435);
+     * N must be a multiple of 4 */
+    MI355Q_SYM128_OUTPUT_BLOCKED = 1
 };
 
 typedef struct {
@@ -147,6 +160,20 @@ int mi355q_q4_weight_prepare(mi355q_context *ctx,
                              int meta_kind, uint32_t flags,
                              mi355q_q4_weight **out,
                              char *error, size_t error_capacity);
+/* Symmetric Q4, group 128 — the tensor format of compiler/q4_image.py that the
+ * portable C runtimes read: per (row, 128-column group) a 66-byte record = bf16
+ * scale then 64 code bytes, element j in byte j/2, even j in the low nibble, the
+ * nibble a two's complement value v in [-8, 7], w = scale * v
+ * (qwen35_task.c:36-38,286-303,426-450).  The records are mapped on the GPU,
+ * without loss, to the affine layout (q = v + 8, bias = -8 * scale, each group
+ * as two 64-column groups), and the returned handle is an ordinary Q4 weight:
+ * every mi355q_q4_linear* entry point takes it.  K must be a non-zero multiple
+ * of 128.  Replaces the record walk of q4_gemv (qwen35_task.c:318-362) and of
+ * linear_grouped (whisper_turbo_encoder.c:127-157). */
+int mi355q_sym128_weight_prepare(mi355q_context *ctx, const void *records,
+                                 uint32_t N, uint32_t K, int record_order,
+                                 uint32_t flags, mi355q_q4_weight **out,
+                                 char *error, size_t error_capacity);
 void mi355q_q4_weight_destroy(mi355q_q4_weight *weight);
 /* Bytes of the original image this weight stands for: N*K/2 + N*(K/64)*4. */
 size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight);
@@ -200,6 +227,34 @@ typedef struct {
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,
                               size_t count, char *error, size_t error_capacity);
+
+/* ---- drop-ins with the reference's own hook signatures ----------------------
+ *
+ * The portable runtimes call their Q4 linear through two compile-time hooks
+ * that take the raw record pointer of the mapped image on every call.  These
+ * two functions have those argument lists (plus an int status where the
+ * reference returns void) and can be bound by a one-line macro or wrapper in the
+ * target's kernel header.  They run on a process-wide context on device 0,
+ * created on first use, and prepare each distinct `weights` pointer once (the
+ * image is mapped read-only for the life of the process, so the pointer
+ * identifies the tensor); activations and outputs are host arrays, fp32.
+ * Status and message of the last failing call: mi355q_hook_last_error.
+ * mi355q_hook_release frees the cached weights and the context. */
+
+/* whisper_turbo_q4_gemm (whisper_turbo_a113x_kernels.h:270-280), called from
+ * linear_any when WHISPER_TURBO_HAVE_Q4_GEMM is defined
+ * (whisper_turbo_encoder.c:160-176): output[r][n] = bias[n] + sum_k w[n][k] *
+ * input[r][k], row-major records, bias may be NULL. */
+int mi355q_hook_q4_gemm(const unsigned char *weights, const float *input, size_t rows,
+                        size_t input_width, size_t output_width, const float *bias,
+                        float *output);
+/* q4_gemv (qwen35_task.c:318-362) with the descriptor's fields passed flat:
+ * output[n] = sum_k w[n][k] * input[k]; record_order as above. */
+int mi355q_hook_q4_gemv(const unsigned char *records, int record_order, size_t rows,
+                        size_t columns, const float *input, float *output);
+int mi355q_hook_last_error(char *message, size_t capacity);
+void mi355q_hook_release(void);
+
 
 /* ---- W8A8: per-token int8 activations x per-output-row int8 weights ---------
  *
