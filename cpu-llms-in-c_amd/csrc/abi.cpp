@@ -308,6 +308,12 @@ int mi355q_q4_weight_prepare(mi355q_context *ctx, const void *quants, const void
         if (status != hipSuccess) break;
         status = hipMalloc((void **)&dev.meta, (size_t)dev.NT * dev.T * 16u * sizeof(uint2));
         if (status != hipSuccess) break;
+        dev.meta16 = dev.meta;
+        if (meta_kind == MI355Q_META_BF16_PLANES) {
+            dev.meta16 = nullptr;
+            status = hipMalloc((void **)&dev.meta16, (size_t)dev.NT * dev.T * 16u * sizeof(uint2));
+            if (status != hipSuccess) break;
+        }
         if (!on_device) {
             what = "image upload";
             status = hipMalloc(&staging, code_bytes + meta_bytes);
@@ -355,6 +361,7 @@ void mi355q_q4_weight_destroy(mi355q_q4_weight *weight)
         (void)hipStreamSynchronize(weight->ctx->stream);
     }
     if (weight->dev.codes) (void)hipFree(weight->dev.codes);
+    if (weight->dev.meta16 && weight->dev.meta16 != weight->dev.meta) (void)hipFree(weight->dev.meta16);
     if (weight->dev.meta) (void)hipFree(weight->dev.meta);
     delete weight;
 }

@@ -37,7 +37,8 @@ constexpr uint32_t kStepColumns = 128;
 
 struct Q4Device {
     uint4 *codes;   // [T][NT][64]
-    uint2 *meta;    // [T][NT][16]
+    uint2 *meta;    // [T][NT][16], fields in the image's own 16-bit encoding
+    uint2 *meta16;  // the same records as fp16 {scale, bias} pairs (== meta for fp16 images): GEMM
     uint32_t N, K;  // logical shape
     uint32_t NT, T; // tiles of 16 rows, steps of 128 columns
     int meta_kind;

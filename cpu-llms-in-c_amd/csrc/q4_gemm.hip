@@ -8,21 +8,28 @@
 // fp32 accumulation over the whole of K.
 //
 // Work split: a workgroup of four waves computes BM (64 or 128) rows of x by
-// 4*NTW (+1) tiles of 16 rows of w: NTW tiles per wave and optionally one more
-// for the last wave.  The host picks the variant whose workgroup count fits the
-// machine (two workgroups per compute unit), e.g. 17 tiles for the 17408-row
-// matrices: 64 x 8 = 512 workgroups at M = 512.  The activations of one 128-column step are staged in
-// LDS by LDS-direct loads (double buffered) and shared by the four waves; every wave dequantizes
-// the codes of its own NTW tiles of 16 weight rows straight into the B-operand
-// registers of the matrix instruction (the stream-tile layout hands each lane
-// exactly the eight consecutive columns the instruction wants), so each weight
-// is dequantized once per workgroup and never passes through LDS.
+// 4*NTW (+1) tiles of 16 rows of w.  The activations of one 128-column step are
+// staged in LDS by LDS-direct loads (double buffered) and shared by the four
+// waves; every wave dequantizes the codes of its own NTW tiles straight into the
+// B-operand registers of the matrix instruction (the stream-tile layout hands
+// each lane exactly the eight consecutive columns the instruction wants), so
+// each weight is dequantized once per workgroup and never passes through LDS.
+// The metadata is read as fp16 {scale, bias} pairs (converted at prepare for
+// bf16 images).  Two kernels:
+//   q4_gemm_kernel: two workgroups per compute unit overlap each other's
+//     dequantization and matrix instructions (six tile shapes);
+//   q4_gemm_pipe_kernel: one workgroup per compute unit, software pipelined by
+//     hand (128 rows x 16 or 17 tiles).
+// The host picks shape and K split by a time estimate fitted on this GPU, e.g.
+// 17 tiles for the 17408-row matrices: 64 x 4 = 256 workgroups at M = 512.
 #include <cstdio>
 #include "device_util.h"
 #include "internal.h"
 
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
+#include <utility>
 
 namespace mi355q {
 
@@ -47,24 +54,66 @@ __device__ __forceinline__ half8 dequant8(uint32_t word, const NibbleMasks &mask
     return __builtin_elementwise_fma(unpack8(word, masks), scale, bias);
 }
 
-template <bool BF>
+// {scale, bias} of one group, both fp16 in one word, broadcast to the eight weights of a lane
 __device__ __forceinline__ void meta_to_half(uint32_t word, half8 &scale, half8 &bias)
 {
-    _Float16 s, b;
-    if (BF) {
-        s = (_Float16)__builtin_bit_cast(float, word << 16);
-        b = (_Float16)__builtin_bit_cast(float, word & 0xffff0000u);
-    } else {
-        s = __builtin_bit_cast(_Float16, (uint16_t)(word & 0xffffu));
-        b = __builtin_bit_cast(_Float16, (uint16_t)(word >> 16));
-    }
+    const _Float16 s = __builtin_bit_cast(_Float16, (uint16_t)(word & 0xffffu));
+    const _Float16 b = __builtin_bit_cast(_Float16, (uint16_t)(word >> 16));
     scale = half8{s, s, s, s, s, s, s, s};
     bias = half8{b, b, b, b, b, b, b, b};
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
+// compile-time constant in the body
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f)
+{
+    (f(std::integral_constant<int, I>()), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>(), f);
+}
+
+// Output of one accumulator fragment: lane (r, kq) holds rows row0 + 4*kq + j (j = 0..3) of
+// column n.  MODE 0..2: plain store as fp16 / fp32 / bf16 (no residual, no K split: the common
+// case, with nothing to decide per element); MODE 3: everything else.
+template <int MODE>
+__device__ __forceinline__ void store_fragment(const GemmParams &p, uint32_t split, uint32_t row0,
+                                               uint32_t kq, uint32_t n, const floatx4 &values)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t m = row0 + 4u * kq + j;
+        if (m >= p.M) continue;
+        const size_t at = (size_t)m * p.N + n;
+        if (MODE == 0) {
+            ((_Float16 *)p.y)[at] = (_Float16)values[j];
+        } else if (MODE == 1) {
+            ((float *)p.y)[at] = values[j];
+        } else if (MODE == 2) {
+            store_from_float(p.y, MI355Q_BF16, at, values[j]);
+        } else if (p.splits > 1u) {
+            p.partials[(size_t)split * p.M * p.N + at] = values[j];
+        } else {
+            float value = values[j];
+            if (p.residual)
+                value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? n : at);
+            store_from_float(p.y, p.y_dtype, at, value);
+        }
+    }
+}
+
+__device__ __forceinline__ int store_mode(const GemmParams &p)
+{
+    if (p.splits > 1u || p.residual != nullptr) return 3;
+    return p.y_dtype == MI355Q_F16 ? 0 : p.y_dtype == MI355Q_F32 ? 1 : 2;
+}
+
 // BM rows of x per workgroup; every wave owns NTW tiles of 16 weight rows and, when EXTRA,
 // the last wave owns one more (tiles per block = 4*NTW + EXTRA).
-template <int BM, int NTW, bool EXTRA, bool BF>
+template <int BM, int NTW, bool EXTRA>
 __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
 {
     // Activation stage: [buffer][row][slot] of 16-byte pieces, slot = octet ^ (row % 16).
@@ -135,7 +184,7 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
     };
     auto dequant_tile = [&](int d, const uint4 &codes, const uint2 &meta, const NibbleMasks &masks) {
         half8 scale, bias;
-        meta_to_half<BF>(d < 2 ? meta.x : meta.y, scale, bias);
+        meta_to_half(d < 2 ? meta.x : meta.y, scale, bias);
         const uint32_t word = d == 0 ? codes.x : d == 1 ? codes.y : d == 2 ? codes.z : codes.w;
         return dequant8(word, masks, scale, bias);
     };
@@ -217,28 +266,269 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
     }
 
     // ---- lane (r, kq) holds rows 16*i + 4*kq + j of column tile*16 + r
+    auto store_all = [&](auto mode) {
 #pragma unroll
-    for (int t = 0; t < NTX; ++t) {
-        if (t == NTW && !has_extra) continue;
-        const uint32_t tile = tile0 + t;
-        const uint32_t n = tile * kTileRows + r;
-        if (tile >= p.NT || n >= p.N) continue;
+        for (int t = 0; t < NTX; ++t) {
+            if (t == NTW && !has_extra) continue;
+            const uint32_t tile = tile0 + t;
+            const uint32_t n = tile * kTileRows + r;
+            if (tile >= p.NT || n >= p.N) continue;
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
+            for (int i = 0; i < MI; ++i)
+                store_fragment<decltype(mode)::value>(p, split, m0 + 16u * i, kq, n, acc[i][t]);
+        }
+    };
+    switch (store_mode(p)) {
+    case 0: store_all(std::integral_constant<int, 0>()); break;
+    case 1: store_all(std::integral_constant<int, 1>()); break;
+    case 2: store_all(std::integral_constant<int, 2>()); break;
+    default: store_all(std::integral_constant<int, 3>()); break;
+    }
+}
+
+// One of the three dependent instructions that dequantize piece PIECE (tile PIECE/4, weights
+// 2*(PIECE%4) and +1 of a lane's eight) of quarter D: mask-and-merge into an fp16 with the code
+// in its mantissa, subtract the offset, fused multiply-add with the group's {scale, bias}.  They
+// are asm statements: asm keeps its source order, which is what places each in its slot between
+// the matrix instructions; the caller keeps dependent stages at least one instruction apart,
+// which covers the wait state a packed-fp16 result needs before a vector instruction reads it.
+template <int STAGE, int PIECE, int D, int NTX>
+__device__ __forceinline__ void dequant_stage(const uint4 (&codes)[NTX], const uint2 (&meta)[NTX],
+                                              const NibbleMasks &masks, uint32_t (&merged)[4 * NTX],
+                                              half2v (&centred)[4 * NTX], half2v (&out)[NTX][4])
+{
+    constexpr int t = PIECE / 4, j = PIECE % 4;
+    if constexpr (STAGE == 0) {
+        uint32_t word = D == 0 ? codes[t].x : D == 1 ? codes[t].y : D == 2 ? codes[t].z : codes[t].w;
+        if (j >= 2) word >>= 8;
+        // fp16 1024 (64) twice, the code in the low (second) mantissa nibble
+        asm volatile("v_and_or_b32 %0, %1, %2, %3"
+                     : "=v"(merged[PIECE])
+                     : "v"(word), "v"((j & 1) ? masks.hi : masks.lo), "s"((j & 1) ? 0x54005400u : 0x64006400u));
+    } else if constexpr (STAGE == 1) {
+        // fp16 -1024 (-64) twice
+        asm volatile("v_pk_add_f16 %0, %1, %2"
+                     : "=v"(centred[PIECE])
+                     : "v"(merged[PIECE]), "s"((j & 1) ? 0xd400d400u : 0xe400e400u));
+    } else {
+        // scale = low half of the metadata word for both results, bias = high half for both
+        asm volatile("v_pk_fma_f16 %0, %1, %2, %2 op_sel:[0,0,1] op_sel_hi:[1,0,1]"
+                     : "=v"(out[t][j])
+                     : "v"(centred[PIECE]), "v"(D < 2 ? meta[t].x : meta[t].y));
+    }
+}
+
+// One workgroup per compute unit, one wave per SIMD, software pipelined: while the
+// matrix instructions of one 32-column quarter run, the same wave dequantizes the
+// next quarter's weights and reads the next quarter's activation fragments from
+// LDS; every matrix instruction is followed by about two vector instructions and,
+// after the last use of a fragment, the LDS read that refills it.
+// With XT the workgroup takes one tile more than its waves can split evenly
+// (4*NTW + 1, e.g. 17 = 1088 / 64): every wave dequantizes that tile and multiplies
+// it with its own quarter of the row fragments, so the four waves stay balanced.
+template <int BM, int NTW, bool XT>
+__global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p)
+{
+    __shared__ uint4 a_lds[2][BM][16];  // [buffer][row][slot], slot = octet ^ (row % 16)
+    constexpr int MI = BM / 16;  // 16-row fragments of x per workgroup
+    constexpr int AJ = BM / 16;  // LDS-direct loads per wave per step (4 rows each)
+    constexpr int TPB = 4 * NTW + (XT ? 1 : 0);
+    constexpr int NTX = NTW + (XT ? 1 : 0);
+    constexpr int XI = MI / 4;  // row fragments of the shared tile per wave
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    typedef const __attribute__((address_space(1))) void *global_ptr;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15u;
+    const uint32_t kq = lane >> 4;
+    const uint32_t m0 = blockIdx.y * BM;
+    const uint32_t tile0 = blockIdx.x * TPB + wave * NTW;
+    const uint32_t shared_tile = blockIdx.x * TPB + 4u * NTW;
+    const uint32_t split = blockIdx.z;
+    const uint32_t step_begin = split * p.steps_per_split;
+    const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
+    if (step_begin >= step_end) return;  // uniform over the workgroup
+
+    // Rows beyond M re-read the last row and columns beyond K re-read the previous group
+    // (finite values against zero weights): both stay in bounds and never reach y.
+    const _Float16 *a_source[AJ];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t m = m0 + 16u * i + 4u * kq + j;
-                if (m >= p.M) continue;
-                const size_t at = (size_t)m * p.N + n;
-                if (p.splits > 1u) {
-                    p.partials[(size_t)split * p.M * p.N + at] = acc[i][t][j];
-                } else {
-                    float value = acc[i][t][j];
-                    if (p.residual)
-                        value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? n : at);
-                    store_from_float(p.y, p.y_dtype, at, value);
-                }
+    for (int j = 0; j < AJ; ++j) {
+        const uint32_t local = (BM / 4) * wave + 4u * j + kq;
+        uint32_t m = m0 + local;
+        m = m < p.M ? m : p.M - 1u;
+        a_source[j] = p.x + (size_t)m * p.K + 8u * (r ^ (local & 15u));
+    }
+    auto fetch_a = [&](uint32_t step, int buffer) {
+#pragma unroll
+        for (int j = 0; j < AJ; ++j) {
+            const uint32_t k = step * kStepColumns;
+            const uint32_t octet = r ^ (((BM / 4) * wave + 4u * j + kq) & 15u);
+            const _Float16 *source = a_source[j] + k;
+            if (k + 8u * octet >= p.K) source -= 64;
+            __builtin_amdgcn_global_load_lds((global_ptr)source,
+                                             (lds_ptr)&a_lds[buffer][(BM / 4) * wave + 4u * j][0], 16, 0, 0);
+        }
+    };
+    auto fetch_tile = [&](uint32_t step, uint32_t tile, uint4 &codes, uint2 &meta) {
+        tile = tile < p.NT ? tile : p.NT - 1u;  // stay in bounds; such columns are never stored
+        const size_t record = (size_t)step * p.NT + tile;
+        codes = p.codes[record * 64u + lane];
+        meta = p.meta[record * 16u + r];
+    };
+    auto fetch_b = [&](uint32_t step, uint4 (&codes)[NTX], uint2 (&meta)[NTX]) {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) fetch_tile(step, tile0 + t, codes[t], meta[t]);
+        if (XT) fetch_tile(step, shared_tile, codes[NTX - 1], meta[NTX - 1]);
+    };
+    const NibbleMasks masks = nibble_masks();
+
+    floatx4 acc[MI][NTW];
+    floatx4 acc_shared[XI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) acc[i][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < XI; ++i) acc_shared[i] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Steady state of one step (buffer = step parity):
+    //   quarters 0..2: matrix instructions of quarter d | LDS reads + dequantization of d+1
+    //   wait for the fetches of step+1, barrier (all waves hold their last fragments of
+    //   this buffer in registers, so it may be refilled)
+    //   quarter 3: fetch step+2 | matrix instructions | reads + dequantization of quarter 0
+    //   of step+1 from the other buffer.
+    // Steps past the end are clamped to the last one (a redundant fetch, no branches).
+    // The matrix instructions are written as asm with the accumulator tied in place (in the
+    // accumulation registers); a scheduling barrier after each pins the few vector
+    // instructions and the LDS read that follow it in the source to that slot.
+    const uint32_t last_step = step_end - 1u;
+    auto clamp_step = [&](uint32_t step) { return step < last_step ? step : last_step; };
+    uint4 b_codes[NTX], next_codes[NTX];
+    uint2 b_meta[NTX], next_meta[NTX];
+    half2v b_frag[2][NTX][4];  // [set][tile][column pair group]: 8 weights of a lane
+    half8 a_frag[MI];
+    half8 a_shared[XI];
+    auto read_frag = [&](int buffer, int d, uint32_t fragment) {
+        return __builtin_bit_cast(half8, a_lds[buffer][16 * fragment + r][(4 * d + kq) ^ r]);
+    };
+    auto multiply = [&](floatx4 &c, const half8 &a, const half2v (&b)[4]) {
+        const half8 b8 = {b[0].x, b[0].y, b[1].x, b[1].y, b[2].x, b[2].y, b[3].x, b[3].y};
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b8));
+    };
+    // Dequantization of one quarter = NTX tiles x 4 pieces (two of a lane's eight weights each),
+    // each piece three dependent vector instructions: mask-and-merge into an fp16 with the code in
+    // its mantissa, subtract the offset, fused multiply-add with the group's {scale, bias}.
+    // Piece p starts in slot p * (SLOTS - 3) / PIECES and advances one stage per slot, so no slot holds two
+    // dependent instructions back to back.
+    constexpr int SLOTS = MI * NTW + (XT ? XI : 0);
+    constexpr int PIECES = 4 * NTX;
+    // The three instructions are asm statements: asm keeps its source order, which is what
+    // places each of them in its slot, and the slot distance between dependent ones also covers
+    // the one wait state a packed-fp16 result needs before the next vector instruction reads it.
+    uint32_t merged[PIECES];
+    half2v centred[PIECES];
+    // One quarter: the matrix instructions on b_frag[cur] and the resident fragments; between
+    // them the dequantization of quarter next_d (of `codes`) into b_frag[cur ^ 1] and the
+    // refill of every fragment, right after its last use, with quarter next_d of next_buffer.
+    auto quarter = [&](auto cur_c, auto next_d_c, int next_buffer, const uint4 (&codes)[NTX],
+                       const uint2 (&meta)[NTX]) {
+        constexpr int cur = decltype(cur_c)::value;
+        static_for<SLOTS>([&](auto k_c) {
+            constexpr int k = decltype(k_c)::value;
+            if constexpr (k < MI * NTW) {
+                constexpr int i = k / NTW, t = k % NTW;
+                multiply(acc[i][t], a_frag[i], b_frag[cur][t]);
+                if constexpr (t == NTW - 1) a_frag[i] = read_frag(next_buffer, decltype(next_d_c)::value, i);
+            } else {
+                constexpr int i = k - MI * NTW;
+                multiply(acc_shared[i], a_shared[i], b_frag[cur][NTX - 1]);
+                a_shared[i] = read_frag(next_buffer, decltype(next_d_c)::value, XI * wave + i);
             }
+            static_for<PIECES>([&](auto piece_c) {
+                constexpr int piece = decltype(piece_c)::value;
+                constexpr int stage = k - piece * (SLOTS - 3) / PIECES;
+                if constexpr (stage >= 0 && stage < 3)
+                    dequant_stage<stage, piece, decltype(next_d_c)::value>(codes, meta, masks, merged,
+                                                                           centred, b_frag[cur ^ 1]);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    fetch_a(step_begin, 0);
+    fetch_b(step_begin, b_codes, b_meta);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    fetch_a(clamp_step(step_begin + 1u), 1);
+    fetch_b(clamp_step(step_begin + 1u), next_codes, next_meta);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a_frag[i] = read_frag(0, 0, i);
+    if (XT) {
+#pragma unroll
+        for (int i = 0; i < XI; ++i) a_shared[i] = read_frag(0, 0, XI * wave + i);
+    }
+    static_for<PIECES>([&](auto piece_c) {
+        static_for<3>([&](auto stage_c) {
+            dequant_stage<decltype(stage_c)::value, decltype(piece_c)::value, 0>(b_codes, b_meta, masks,
+                                                                                  merged, centred, b_frag[0]);
+            asm volatile("s_nop 1");  // packed-fp16 result to its reader: one wait state
+        });
+    });
+
+    for (uint32_t step = step_begin; step < step_end; ++step) {
+        const int buffer = (int)((step - step_begin) & 1u);
+        static_for<3>([&](auto d_c) {
+            constexpr int d = decltype(d_c)::value;
+            __builtin_amdgcn_sched_barrier(0);
+            quarter(std::integral_constant<int, (d & 1)>(), std::integral_constant<int, d + 1>(), buffer,
+                    b_codes, b_meta);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): fetches landed, LDS reads done
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_a(clamp_step(step + 2u), buffer);
+        quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), buffer ^ 1, next_codes,
+                next_meta);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NTX; ++t) {
+            b_codes[t] = next_codes[t];
+            b_meta[t] = next_meta[t];
+        }
+        fetch_b(clamp_step(step + 2u), next_codes, next_meta);
+    }
+
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the last step's spare fetch into LDS has landed
+
+    // ---- lane (r, kq) holds rows 16*i + 4*kq + j of column tile*16 + r
+    auto store_all = [&](auto mode) {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) {
+            const uint32_t tile = tile0 + t;
+            const uint32_t n = tile * kTileRows + r;
+            if (tile >= p.NT || n >= p.N) continue;
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+                store_fragment<decltype(mode)::value>(p, split, m0 + 16u * i, kq, n, acc[i][t]);
+        }
+        if (XT) {
+            const uint32_t n = shared_tile * kTileRows + r;
+            if (shared_tile < p.NT && n < p.N) {
+#pragma unroll
+                for (int i = 0; i < XI; ++i)
+                    store_fragment<decltype(mode)::value>(p, split, m0 + 16u * (XI * wave + i), kq, n,
+                                                          acc_shared[i]);
+            }
+        }
+    };
+    switch (store_mode(p)) {
+    case 0: store_all(std::integral_constant<int, 0>()); break;
+    case 1: store_all(std::integral_constant<int, 1>()); break;
+    case 2: store_all(std::integral_constant<int, 2>()); break;
+    default: store_all(std::integral_constant<int, 3>()); break;
     }
 }
 
@@ -273,7 +563,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     GemmParams p;
     memset(&p, 0, sizeof p);
     p.codes = w.codes;
-    p.meta = w.meta;
+    p.meta = w.meta16;  // fp16 {scale, bias}: the weight is evaluated in fp16 here
     p.x = (const _Float16 *)a.x;
     if (a.x_dtype != MI355Q_F16) {
         const size_t count = (size_t)a.M * w.K;
@@ -308,9 +598,12 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         int resident;          // workgroups that fit one compute unit (registers, LDS)
         double alone, shared;  // fraction of matrix-instruction peak, one / several per CU
     };
-    static const Variant variants[] = {{128, 4, 0, 2, 0.384, 0.482}, {128, 2, 0, 2, 0.301, 0.407},
-                                       {64, 4, 0, 3, 0.309, 0.429},  {64, 4, 1, 2, 0.322, 0.438},
-                                       {64, 2, 0, 4, 0.300, 0.397},  {64, 2, 1, 2, 0.300, 0.441}};
+    // 0-5: two workgroups per compute unit overlap each other; 6, 7: the pipelined kernel,
+    // one workgroup per compute unit
+    static const Variant variants[] = {{128, 4, 0, 2, 0.407, 0.495}, {128, 2, 0, 2, 0.346, 0.451},
+                                       {64, 4, 0, 3, 0.354, 0.464},  {64, 4, 1, 2, 0.384, 0.478},
+                                       {64, 2, 0, 4, 0.350, 0.428},  {64, 2, 1, 2, 0.399, 0.469},
+                                       {128, 4, 0, 1, 0.449, 0.360}, {128, 4, 1, 1, 0.429, 0.373}};
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     int best = 0;
     uint32_t best_splits = 1;
@@ -327,16 +620,18 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             const uint64_t groups = (uint64_t)n_blocks * m_blocks * splits;
             // one workgroup at peak: 64 matrix-instruction cycles per (tile, 16-row
             // fragment, step) and wave, at 2.4 GHz
-            const double peak_us = (double)steps * (c.ntw + c.extra) * (c.bm / 16.0) * 64.0 / 2400.0;
+            // (the pipelined kernel spreads its odd tile over the four waves)
+            const double tiles_per_wave = v >= 6 ? c.ntw + 0.25 * c.extra : c.ntw + c.extra;
+            const double peak_us = (double)steps * tiles_per_wave * (c.bm / 16.0) * 64.0 / 2400.0;
             double cost;
             if (groups <= cus)
                 cost = peak_us / c.alone;
             else if (groups <= slots)
                 cost = (double)((groups + cus - 1) / cus) * peak_us / c.shared;
             else
-                cost = ((double)groups / slots + 0.3) * c.resident * peak_us / c.shared;
+                cost = ((double)groups / slots + 0.315) * c.resident * peak_us / c.shared;
             if (splits > 1)  // fp32 partials written and read back
-                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.9e12 * 1.0e6;
+                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.5e12 * 1.0e6;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;
@@ -370,19 +665,17 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         p.partials = (float *)ctx->stage[4];
     }
     const dim3 grid(n_blocks, m_blocks, p.splits);
-    const bool bf = w.meta_kind == MI355Q_META_BF16_PLANES;
     hipError_t launched = hipErrorInvalidValue;
-#define MI355Q_GEMM_CASE(index, BM, NTW, EXTRA)                                                 \
-    if (best == index)                                                                         \
-        launched = bf ? launch(ctx, q4_gemm_kernel<BM, NTW, EXTRA, true>, grid, dim3(256), 0, p) \
-                      : launch(ctx, q4_gemm_kernel<BM, NTW, EXTRA, false>, grid, dim3(256), 0, p);
-    MI355Q_GEMM_CASE(0, 128, 4, false)
-    MI355Q_GEMM_CASE(1, 128, 2, false)
-    MI355Q_GEMM_CASE(2, 64, 4, false)
-    MI355Q_GEMM_CASE(3, 64, 4, true)
-    MI355Q_GEMM_CASE(4, 64, 2, false)
-    MI355Q_GEMM_CASE(5, 64, 2, true)
-#undef MI355Q_GEMM_CASE
+    switch (best) {
+    case 0: launched = launch(ctx, q4_gemm_kernel<128, 4, false>, grid, dim3(256), 0, p); break;
+    case 1: launched = launch(ctx, q4_gemm_kernel<128, 2, false>, grid, dim3(256), 0, p); break;
+    case 2: launched = launch(ctx, q4_gemm_kernel<64, 4, false>, grid, dim3(256), 0, p); break;
+    case 3: launched = launch(ctx, q4_gemm_kernel<64, 4, true>, grid, dim3(256), 0, p); break;
+    case 4: launched = launch(ctx, q4_gemm_kernel<64, 2, false>, grid, dim3(256), 0, p); break;
+    case 5: launched = launch(ctx, q4_gemm_kernel<64, 2, true>, grid, dim3(256), 0, p); break;
+    case 6: launched = launch(ctx, q4_gemm_pipe_kernel<128, 4, false>, grid, dim3(256), 0, p); break;
+    default: launched = launch(ctx, q4_gemm_pipe_kernel<128, 4, true>, grid, dim3(256), 0, p); break;
+    }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);
     if (p.splits > 1u) {

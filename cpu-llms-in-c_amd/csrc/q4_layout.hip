@@ -42,8 +42,8 @@ q4_repack_codes_kernel(const uint32_t *__restrict__ src_words, uint4 *__restrict
 __global__ void __launch_bounds__(256)
 q4_repack_meta_kernel(const uint16_t *__restrict__ meta_a,
                       const uint16_t *__restrict__ meta_b, int meta_kind,
-                      uint2 *__restrict__ dst, uint32_t N, uint32_t K, uint32_t NT,
-                      uint32_t T)
+                      uint2 *__restrict__ dst, uint2 *__restrict__ dst16, uint32_t N, uint32_t K,
+                      uint32_t NT, uint32_t T)
 {
     uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint64_t total = (uint64_t)NT * T * 16u;
@@ -74,6 +74,16 @@ q4_repack_meta_kernel(const uint16_t *__restrict__ meta_a,
         out[h] = value;
     }
     dst[index] = make_uint2(out[0], out[1]);
+    if (dst16 != nullptr) {  // bf16 image: an fp16 copy for the matrix-instruction GEMM
+#pragma unroll
+        for (uint32_t h = 0; h < 2; ++h) {
+            const _Float16 scale = (_Float16)__builtin_bit_cast(float, out[h] << 16);
+            const _Float16 bias = (_Float16)__builtin_bit_cast(float, out[h] & 0xffff0000u);
+            out[h] = (uint32_t)__builtin_bit_cast(uint16_t, scale) |
+                     ((uint32_t)__builtin_bit_cast(uint16_t, bias) << 16);
+        }
+        dst16[index] = make_uint2(out[0], out[1]);
+    }
 }
 
 // Symmetric group-128 records (bf16 scale + 64 code bytes, two's complement
@@ -130,7 +140,8 @@ hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
     hipLaunchKernelGGL(q4_repack_codes_kernel, dim3(code_blocks), dim3(256), 0, stream,
                        codes_src, dst.codes, dst.N, dst.K, dst.NT, dst.T);
     hipLaunchKernelGGL(q4_repack_meta_kernel, dim3(meta_blocks), dim3(256), 0, stream,
-                       meta_a, meta_b, dst.meta_kind, dst.meta, dst.N, dst.K, dst.NT,
+                       meta_a, meta_b, dst.meta_kind, dst.meta,
+                       dst.meta16 != dst.meta ? dst.meta16 : (uint2 *)nullptr, dst.N, dst.K, dst.NT,
                        dst.T);
     return hipGetLastError();
 }
