@@ -71,7 +71,7 @@ def q4_bytes(N, K, M, y_bytes=2):
     return N * K // 2 + N * (K // 64) * 4 + M * K * 2 + M * N * y_bytes
 
 
-def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True):
+def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True, silu=False):
     """Prepares `copies` device copies of every matrix plus activations/outputs."""
     x_ptr, y_ptr, weights, host = {}, {}, [[] for _ in range(copies)], {}
     for index, (name, N, K) in enumerate(shapes):
@@ -99,8 +99,11 @@ def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True
                 groups[-1][0].append(target)
             else:
                 groups.append(([target], K))
-        calls.append(engine.make_calls([(targets, x_ptr[K], engine.F16, M, engine.F16)
-                                        for targets, K in groups]))
+        # --fused-mlp: the gate|up launch writes silu(gate . x) * (up . x) into gate's output
+        calls.append(engine.make_calls([
+            (targets, x_ptr[K], engine.F16, M, engine.F16, engine.F32,
+             engine.FUSE_GATE_UP_SILU if silu and len(targets) == 2 else 0)
+            for targets, K in groups]))
     return calls, weights, host, x_ptr, y_ptr
 
 
@@ -328,6 +331,8 @@ def main():
     parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "prefill", "w8a8"])
     parser.add_argument("--unfused", action="store_true",
                         help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
+    parser.add_argument("--fused-mlp", action="store_true",
+                        help="gate|up launch applies silu(gate)*up (one output instead of two)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args()
@@ -352,7 +357,8 @@ def main():
     ctx = engine.Context(0)  # raises without a GPU
     info = ctx.info()
     calls, weights, host, x_ptr, y_ptr = build_workload(engine, ctx, shapes, M, copies, meta_kind,
-                                                        args.verbose, fuse=not args.unfused)
+                                                        args.verbose, fuse=not args.unfused,
+                                                        silu=args.fused_mlp)
     launches_per_step = len(calls[0])
     step_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
 
@@ -403,6 +409,7 @@ def main():
                         else "affine-Q4 g64 GEMV K=1024 N=3584 M=%d, fp16 scale+bias, fp16 x and y" % M,
             "linears_per_step": len(shapes),
             "launches_per_step": launches_per_step,
+            "gate_up_silu_fused": bool(args.fused_mlp),
             "algorithmic_bytes_per_step": step_bytes,
             "weight_copies_rotated": copies,
             "rotated_bytes": step_bytes * copies,

@@ -433,10 +433,11 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
                   kMaxTargets);
         return MI355Q_ERROR_INVALID;
     }
+    const bool fuse = (flags & MI355Q_FUSE_GATE_UP_SILU) != 0;
     bool any_residual = false;
     for (uint32_t t = 0; t < count; ++t) {
         const mi355q_q4_target &target = targets[t];
-        if (target.weight == nullptr || target.y == nullptr) {
+        if (target.weight == nullptr || (target.y == nullptr && !(fuse && t == 1))) {
             set_error(error, error_capacity, "q4_linear: null weight or output (target %u)", t);
             return MI355Q_ERROR_INVALID;
         }
@@ -458,6 +459,17 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
                   M, x_dtype, y_dtype, residual_dtype);
         return MI355Q_ERROR_INVALID;
     }
+    if (fuse) {
+        const uint32_t rows = x_dtype == MI355Q_F32 ? 2u * M : M;
+        if (count != 2 || targets[0].weight->dev.N != targets[1].weight->dev.N || any_residual ||
+            rows > 16u) {
+            set_error(error, error_capacity,
+                      "q4_linear: gate-up-silu needs two weights of equal shape, no residual and at "
+                      "most 16 activation rows (8 of fp32)");
+            return MI355Q_ERROR_INVALID;
+        }
+    }
+    const uint32_t outputs = fuse ? 1u : count;  // targets whose y is written
     const bool x_dev = flags & MI355Q_X_DEVICE, y_dev = flags & MI355Q_Y_DEVICE;
     const bool r_dev = !any_residual || (flags & MI355Q_RESIDUAL_DEVICE);
     const bool is_bias = (flags & MI355Q_RESIDUAL_IS_BIAS) != 0;
@@ -492,6 +504,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
     args.y_dtype = y_dtype;
     args.residual_dtype = residual_dtype;
     args.residual_is_bias = is_bias;
+    args.fuse_silu = fuse;
     args.count = count;
     int status;
     if (!x_dev) {
@@ -530,7 +543,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
     if (status != MI355Q_OK) return status;
 
     if (!y_dev)
-        for (uint32_t t = 0; t < count; ++t)
+        for (uint32_t t = 0; t < outputs; ++t)
             MI355Q_HIP(hipMemcpyAsync(targets[t].y, args.targets[t].y,
                                       (size_t)M * targets[t].weight->dev.N * dtype_bytes(y_dtype),
                                       hipMemcpyDeviceToHost, ctx->stream),
@@ -560,8 +573,9 @@ int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, 
     for (size_t i = 0; i < count; ++i) {
         const mi355q_q4_call &c = calls[i];
         char inner[256] = "";
+        const uint32_t own = c.flags & (MI355Q_RESIDUAL_IS_BIAS | MI355Q_FUSE_GATE_UP_SILU);
         int status = mi355q_q4_linear_multi(ctx, c.targets, c.target_count, c.x, c.x_dtype, c.M,
-                                            c.y_dtype, c.residual_dtype, flags, inner, sizeof inner);
+                                            c.y_dtype, c.residual_dtype, flags | own, inner, sizeof inner);
         if (status != MI355Q_OK) {
             set_error(error, error_capacity, "call %zu: %s", i, inner);
             return status;

@@ -136,6 +136,7 @@ struct Q4LinearArgs {
     int y_dtype;
     int residual_dtype;
     bool residual_is_bias;  // residual is one row [N] added to every activation row
+    bool fuse_silu;         // targets = {gate, up}: y[0] = silu(gate . x) * (up . x)
     uint32_t count;
     Q4Target targets[kMaxTargets];
 };

@@ -54,8 +54,18 @@ struct StreamParams {
     int pair;
     int y_dtype, residual_dtype;
     int residual_is_bias;  // residual is one row [N], added to every activation row
+    // two targets (gate, up) of equal shape: a workgroup takes TB/2 tiles of each and writes
+    // y[0] = silu(gate . x) * (up . x)
+    int fuse_silu;
     int meta_bf16;
 };
+
+// silu(gate) * up as the reference's fused kernel evaluates it (qwen38_q4.metal:129-151):
+// gate / (1 + exp(-gate)) * up in fp32
+__device__ __forceinline__ float silu_times(float gate, float up)
+{
+    return gate / (1.0f + __expf(-gate)) * up;
+}
 
 template <int TB>
 struct StepData {
@@ -78,7 +88,9 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     for (uint32_t t = 1; t < kMaxTargets; ++t)
         if (t < p.targets && blockIdx.x >= p.first_block[t]) target = t;
     const uint32_t NT = p.NT[target], N = p.N[target];
-    const uint32_t tile0 = (blockIdx.x - p.first_block[target]) * TB;
+    // tiles per target and workgroup: TB, or TB/2 of each of the two fused targets
+    const uint32_t span_tiles = p.fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
+    const uint32_t tile0 = (blockIdx.x - p.first_block[target]) * span_tiles;
 
     uint4 *xs = lds;                                                 // [chunk octets][MP]
     float *red = (float *)(lds + (size_t)p.chunk_steps * 16u * MP);  // [W][TB][NJ][64]
@@ -89,10 +101,11 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint2 *meta_tile[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
-        uint32_t tile = tile0 + tb;
+        const uint32_t slot_target = p.fuse_silu ? (uint32_t)tb / span_tiles : target;
+        uint32_t tile = tile0 + (uint32_t)tb % span_tiles;
         tile = tile < NT ? tile : NT - 1u;
-        codes_tile[tb] = p.codes[target] + (size_t)tile * 64u + lane;
-        meta_tile[tb] = p.meta[target] + (size_t)tile * 16u + r;
+        codes_tile[tb] = p.codes[slot_target] + (size_t)tile * 64u + lane;
+        meta_tile[tb] = p.meta[slot_target] + (size_t)tile * 16u + r;
     }
 
     floatx4 acc[TB];
@@ -215,33 +228,46 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     __syncthreads();
     for (uint32_t e = threadIdx.x; e < TB * 64u; e += 64u * W) {
         const uint32_t tb = e >> 6, l = e & 63u;
-        const uint32_t tile = tile0 + tb;
+        const uint32_t slot_target = p.fuse_silu ? tb / span_tiles : target;
+        const uint32_t tile = tile0 + tb % span_tiles;
         const uint32_t n = tile * kTileRows + (l & 15u);
         if (tile >= NT || n >= N) continue;
-        float v[NJ];
+        const bool fuse_here = p.fuse_silu && p.slices <= 1u;  // else the reduction kernel fuses
+        if (fuse_here && tb >= span_tiles) continue;           // the gate slot's thread does both
+        float v[NJ], up[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            float sum = 0.0f;
+            float sum = 0.0f, sum_up = 0.0f;
 #pragma unroll
             for (int w = 0; w < W; ++w) sum += red[((w * TB + tb) * NJ + j) * 64u + l];
+            if (fuse_here) {
+#pragma unroll
+                for (int w = 0; w < W; ++w) sum_up += red[((w * TB + tb + span_tiles) * NJ + j) * 64u + l];
+            }
             v[j] = sum;
+            up[j] = sum_up;
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const uint32_t row = 4u * (l >> 4) + j;
             if (row >= p.rows) continue;
-            float value = v[j];
+            float value = v[j], value_up = up[j];
             uint32_t m = row;
             if (p.pair) {
                 if (j & 1) continue;
                 value += v[(j + 1) % NJ];
+                value_up += up[(j + 1) % NJ];
                 m = row >> 1;
             }
             if (p.slices > 1u) {
-                p.partials[((size_t)blockIdx.y * p.M + m) * p.n_total + p.n_first[target] + n] = value;
+                p.partials[((size_t)blockIdx.y * p.M + m) * p.n_total + p.n_first[slot_target] + n] = value;
                 continue;
             }
             const size_t at = (size_t)m * N + n;
+            if (fuse_here) {
+                store_from_float(p.y[0], p.y_dtype, at, silu_times(value, value_up));
+                continue;
+            }
             if (p.residual[target])
                 value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
             store_from_float(p.y[target], p.y_dtype, at, value);
@@ -265,6 +291,14 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
         value += p.partials[((size_t)s * p.M + m) * p.n_total + column];
     const uint32_t n = column - p.n_first[target];
     const size_t at = (size_t)m * p.N[target] + n;
+    if (p.fuse_silu) {  // columns [0, N) hold gate . x, [N, 2N) hold up . x
+        if (target != 0u) return;
+        float value_up = 0.0f;
+        for (uint32_t s = 0; s < p.slices; ++s)
+            value_up += p.partials[((size_t)s * p.M + m) * p.n_total + p.n_first[1] + n];
+        store_from_float(p.y[0], p.y_dtype, at, silu_times(value, value_up));
+        return;
+    }
     if (p.residual[target])
         value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
     store_from_float(p.y[target], p.y_dtype, at, value);
@@ -309,7 +343,10 @@ template <int MP, int TB, int D, int W>
 static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
 {
     uint32_t blocks = 0;
-    for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
+    if (p.fuse_silu)
+        blocks = (p.NT[0] + (TB > 1 ? TB / 2 : 1) - 1) / (TB > 1 ? TB / 2 : 1);
+    else
+        for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
     const size_t lds = stream_lds_bytes(MP, TB, W, p.chunk_steps);
     const dim3 grid(blocks, p.slices);
     if (p.meta_bf16)
@@ -418,7 +455,8 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     }
     uint32_t tiles = 0;
     for (uint32_t t = 0; t < a.count; ++t) tiles += a.targets[t].w->NT;
-    const StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
+    StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
+    if (a.fuse_silu && shape.tb != 2 && shape.tb != 4) shape.tb = 2;  // gate and up tiles pair up
     uint32_t block = 0;
     for (uint32_t t = 0; t < a.count; ++t) {
         const Q4Device &w = *a.targets[t].w;
@@ -431,6 +469,8 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         p.first_block[t] = block;
         block += (w.NT + shape.tb - 1) / shape.tb;
     }
+    if (a.fuse_silu) p.first_block[1] = 0xffffffffu;  // every workgroup starts from target 0
+    p.fuse_silu = a.fuse_silu;
     p.targets = a.count;
     p.M = a.M;
     p.K = first.K;

@@ -20,6 +20,7 @@ OK, ERROR_RUNTIME, ERROR_INVALID = 0, 1, 2
 F16, F32, BF16 = 0, 1, 2
 META_F16_INTERLEAVED, META_BF16_PLANES = 0, 1
 X_DEVICE, Y_DEVICE, RESIDUAL_DEVICE, ASYNC, SOURCE_DEVICE, RESIDUAL_IS_BIAS = 1, 2, 4, 8, 16, 32
+FUSE_GATE_UP_SILU = 64
 SYM128_ROW_MAJOR, SYM128_OUTPUT_BLOCKED = 0, 1
 
 _c = ctypes
@@ -48,7 +49,8 @@ class Q4Target(_c.Structure):
 
 class Q4Call(_c.Structure):
     _fields_ = [("x", _vp), ("M", _u32), ("x_dtype", _int), ("y_dtype", _int),
-                ("residual_dtype", _int), ("target_count", _u32), ("targets", Q4Target * 4)]
+                ("residual_dtype", _int), ("target_count", _u32), ("targets", Q4Target * 4),
+                ("flags", _u32)]
 
 
 # name -> (restype, argtypes): every symbol the two headers declare
@@ -251,6 +253,19 @@ class Context:
               RESIDUAL_IS_BIAS if residual_is_bias else 0)
         return y
 
+    def q4_gate_up_silu(self, gate: Q4Weight, up: Q4Weight, x: np.ndarray, x_dtype: int,
+                        y_dtype: int = F32) -> np.ndarray:
+        """Host-array form of the fused call: silu(gate . x) * (up . x), [M][N]."""
+        x = np.ascontiguousarray(x)
+        M = x.shape[0]
+        y = np.empty((M, gate.N), dtype=_NP_DTYPE[y_dtype])
+        targets = (Q4Target * 2)()
+        targets[0].weight, targets[0].y = gate.handle, y.ctypes.data
+        targets[1].weight = up.handle
+        _call(self.lib.mi355q_q4_linear_multi, self.handle, targets, 2, _ptr(x), x_dtype, M, y_dtype, F32,
+              FUSE_GATE_UP_SILU)
+        return y
+
     def q4_linear_multi(self, weights, x: np.ndarray, x_dtype: int, y_dtype: int = F32):
         """Host-array form of the shared-x call: returns one y per weight."""
         x = np.ascontiguousarray(x)
@@ -313,7 +328,7 @@ class Context:
 
 
 def make_calls(items):
-    """items: iterable of (targets, x_ptr, x_dtype, M, y_dtype[, residual_dtype]) where targets is
+    """items: iterable of (targets, x_ptr, x_dtype, M, y_dtype[, residual_dtype[, flags]]) where targets is
     a Q4Weight with its y pointer `(weight, y_ptr[, residual_ptr])` or a list of up to four of them
     (one launch, shared x)."""
     items = list(items)
@@ -324,6 +339,7 @@ def make_calls(items):
             targets = [targets]
         slot.x, slot.M, slot.x_dtype, slot.y_dtype = x_ptr, M, x_dtype, y_dtype
         slot.residual_dtype = item[5] if len(item) > 5 else F32
+        slot.flags = item[6] if len(item) > 6 else 0
         slot.target_count = len(targets)
         for index, target in enumerate(targets):
             slot.targets[index].weight = target[0].handle

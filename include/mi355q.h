@@ -67,7 +67,13 @@ enum {
     MI355Q_SOURCE_DEVICE = 1u << 4,   /* prepare: image pointers are device pointers */
     /* the residual is one row [N] added to every activation row: the `bias` of the
      * reference's grouped linear (whisper_turbo_encoder.c:127-157) */
-    MI355Q_RESIDUAL_IS_BIAS = 1u << 5
+    MI355Q_RESIDUAL_IS_BIAS = 1u << 5,
+    /* mi355q_q4_linear_multi with exactly two targets {gate, up} of equal shape and at most
+     * 16 activation rows (8 when x is fp32): targets[0].y = silu(gate . x) * (up . x),
+     * silu(g) = g / (1 + exp(-g)) in fp32; targets[1].y is not written and may be NULL; no
+     * residuals.  The reference's fused decode kernel qwen38_q4_gate_up_silu
+     * (qwen38_q4.metal:129-151; source_mlp_reference_first_8, qwen38_m3_pack.c:244-349) */
+    MI355Q_FUSE_GATE_UP_SILU = 1u << 6
 };
 
 /* record order of a symmetric group-128 Q4 tensor */
@@ -223,6 +229,7 @@ typedef struct {
     int x_dtype, y_dtype, residual_dtype;
     uint32_t target_count; /* 1..4 */
     mi355q_q4_target targets[4];
+    uint32_t flags; /* MI355Q_RESIDUAL_IS_BIAS, MI355Q_FUSE_GATE_UP_SILU or 0 */
 } mi355q_q4_call;
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,

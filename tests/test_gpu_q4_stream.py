@@ -153,3 +153,44 @@ def test_shared_activation_multi_launch(engine, oracle, gpu, M):
     finally:
         for w in weights:
             w.destroy()
+
+
+@pytest.mark.parametrize("N,K,M,x_dtype", [(1000, 1536, 1, "F16"), (1000, 1536, 3, "F16"),
+                                           (2048, 1024, 8, "BF16"), (640, 8704, 8, "F16"),
+                                           (640, 8704, 4, "F32"), (17408, 5120, 1, "F16")])
+def test_fused_gate_up_silu(engine, oracle, gpu, N, K, M, x_dtype):
+    """MI355Q_FUSE_GATE_UP_SILU: y = silu(gate . x) * (up . x) in one launch
+    (qwen38_q4_gate_up_silu, qwen38_q4.metal:129-151), against the oracle's two exact-weight dots
+    combined in float64; (640, 8704) is cut in K slices, so the reduction kernel applies the
+    nonlinearity there.  Also through the sequence call, with device pointers."""
+    x_dtype = getattr(engine, x_dtype)
+    gate_image = engine.synth_q4_affine(21, 0.02, N, K, engine.META_BF16_PLANES)
+    up_image = engine.synth_q4_affine(22, 0.02, N, K, engine.META_BF16_PLANES)
+    x = make_x(engine, 23, M, K, x_dtype)
+    gate = gpu.q4_prepare(*gate_image, N, K, engine.META_BF16_PLANES)
+    up = gpu.q4_prepare(*up_image, N, K, engine.META_BF16_PLANES)
+    x_ptr = y_ptr = None
+    try:
+        print(f"fused case N={N} K={K} M={M} x={x_dtype}", flush=True)
+        y = gpu.q4_gate_up_silu(gate, up, x, x_dtype, engine.F32)
+        x_ptr, y_ptr = gpu.to_device(x), gpu.alloc(M * N * 4)
+        calls = engine.make_calls([([(gate, y_ptr), (up, None)], x_ptr, x_dtype, M, engine.F32, engine.F32,
+                                    engine.FUSE_GATE_UP_SILU)])
+        gpu.q4_sequence(calls)
+        gpu.sync()
+        queued = gpu.download(y_ptr, (M, N), np.float32)
+        with pytest.raises(engine.Mi355qError) as info:  # three targets cannot be fused
+            gpu.q4_sequence(engine.make_calls([([(gate, y_ptr), (up, y_ptr), (up, y_ptr)], x_ptr, x_dtype, M,
+                                                engine.F32, engine.F32, engine.FUSE_GATE_UP_SILU)]))
+        assert info.value.status == engine.ERROR_INVALID
+    finally:
+        for pointer in (x_ptr, y_ptr):
+            if pointer:
+                gpu.free(pointer)
+        gate.destroy()
+        up.destroy()
+    g = oracle.q4_linear(*gate_image, engine.META_BF16_PLANES, N, K, x, x_dtype, M)
+    u = oracle.q4_linear(*up_image, engine.META_BF16_PLANES, N, K, x, x_dtype, M)
+    reference = g / (1.0 + np.exp(-g)) * u
+    assert q4_relative_error(y, reference) <= TOLERANCE
+    assert np.array_equal(y.view(np.uint32), queued.view(np.uint32))
