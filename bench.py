@@ -107,6 +107,17 @@ def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True
     return calls, weights, host, x_ptr, y_ptr
 
 
+def weights_digest(host, shapes):
+    """SHA-256 over the packed synthetic weights (codes, then metadata planes, matrix by matrix)."""
+    import hashlib
+    digest = hashlib.sha256()
+    for name, _, _ in shapes:
+        for plane in host[name]:
+            if plane is not None:
+                digest.update(np.ascontiguousarray(plane).view(np.uint8))
+    return digest.hexdigest()
+
+
 def cpu_baseline(oracle, shapes, host, M, meta_kind, repeats=5):
     """The oracle's reference-faithful flavour (fp32, k order) on all host threads."""
     threads = min(os.cpu_count() or 1, 16)
@@ -122,8 +133,15 @@ def cpu_baseline(oracle, shapes, host, M, meta_kind, repeats=5):
         if rep:
             times.append(time.perf_counter() - t0)
     median = sorted(times)[len(times) // 2]
+    t0 = time.perf_counter()  # the reference's deployment width: four threads (one pass)
+    for name, N, K in shapes:
+        quants, meta_a, meta_b = host[name]
+        oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, host[("x", K)], oracle.X_F16,
+                         M, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=4)
+    four = time.perf_counter() - t0
     return {
         "value": round(total_bytes / median / 1e9, 3),
+        "value_at_4_threads": round(total_bytes / four / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
@@ -379,6 +397,10 @@ def main():
     ctx.profile_begin()
     run_steps(args.steps)
     kernel_ms, launches = ctx.profile_end()
+    per_launch = ctx.profile_durations()
+    # kernel time of each step (its launches, and the slice reductions some of them carry)
+    per_step = per_launch[:len(per_launch) // args.steps * args.steps].reshape(args.steps, -1).sum(axis=1)
+    p10, p50, p90 = (float(np.percentile(per_step, q)) for q in (10, 50, 90))
 
     # measured plain-read ceiling: whole 2 GiB pass, and launches the size of one weight matrix
     read_long = ctx.probe_read_bandwidth(2 << 30, 3, 1, 0)
@@ -415,6 +437,9 @@ def main():
             "rotated_bytes": step_bytes * copies,
             "percent_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
             "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
+            "kernel_us_per_step_p10_p50_p90": [round(p10, 2), round(p50, 2), round(p90, 2)],
+            "gb_per_s_at_p50_kernel_time": round(step_bytes / (p50 * 1e-6) / 1e9, 1),
+            "weights_sha256": weights_digest(host, shapes),
             "device": info.name.decode(errors="replace").strip(),
             "arch": info.arch.decode(errors="replace"),
             "compute_units": info.compute_units,

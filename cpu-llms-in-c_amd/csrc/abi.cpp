@@ -249,6 +249,24 @@ int mi355q_profile_end(mi355q_context *ctx, double *kernel_ms, uint64_t *launche
     return MI355Q_OK;
 }
 
+int mi355q_profile_durations(mi355q_context *ctx, double *kernel_us, size_t capacity, size_t *count,
+                             char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || count == nullptr || ctx->profiling || (kernel_us == nullptr && capacity != 0)) {
+        set_error(error, error_capacity, "profile_durations: call after profile_end, with a count");
+        return MI355Q_ERROR_INVALID;
+    }
+    const size_t launches = ctx->profile_used / 2;
+    *count = launches;
+    for (size_t i = 0; i < launches && i < capacity; ++i) {
+        float ms = 0.0f;
+        MI355Q_HIP(hipEventElapsedTime(&ms, (*ctx->profile_events)[2 * i], (*ctx->profile_events)[2 * i + 1]),
+                   "hipEventElapsedTime");
+        kernel_us[i] = (double)ms * 1.0e3;
+    }
+    return MI355Q_OK;
+}
+
 // ---- affine Q4 ---------------------------------------------------------------
 
 int mi355q_q4_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,

@@ -67,6 +67,7 @@ SIGNATURES = {
     "mi355q_timer_end": (_int, [_vp, _c.POINTER(_c.c_double), *_err]),
     "mi355q_profile_begin": (_int, [_vp, *_err]),
     "mi355q_profile_end": (_int, [_vp, _c.POINTER(_c.c_double), _c.POINTER(_u64), *_err]),
+    "mi355q_profile_durations": (_int, [_vp, _vp, _sz, _c.POINTER(_sz), *_err]),
     "mi355q_probe_read_bandwidth": (_int, [_vp, _sz, _sz, _int, _int, _c.POINTER(_c.c_double), *_err]),
     "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
                                         _c.POINTER(_vp), *_err]),
@@ -218,6 +219,14 @@ class Context:
         ms, launches = ctypes.c_double(), ctypes.c_uint64()
         _call(self.lib.mi355q_profile_end, self.handle, ctypes.byref(ms), ctypes.byref(launches))
         return ms.value, launches.value
+
+    def profile_durations(self) -> np.ndarray:
+        """Per-launch kernel durations (us) of the profile that just ended, in launch order."""
+        count = ctypes.c_size_t()
+        _call(self.lib.mi355q_profile_durations, self.handle, None, 0, ctypes.byref(count))
+        out = np.empty(count.value, dtype=np.float64)
+        _call(self.lib.mi355q_profile_durations, self.handle, _ptr(out), out.size, ctypes.byref(count))
+        return out
 
     def probe_read_bandwidth(self, nbytes: int = 2 << 30, repeats: int = 5, variant: int = 1,
                              launch_bytes: int = 0) -> float:

@@ -137,6 +137,10 @@ int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms,
 int mi355q_profile_begin(mi355q_context *ctx, char *error, size_t error_capacity);
 int mi355q_profile_end(mi355q_context *ctx, double *kernel_ms, uint64_t *launches,
                        char *error, size_t error_capacity);
+/* After mi355q_profile_end: the individual durations, in launch order, of the kernels the
+ * last profile covered (`count` = how many there were; at most `capacity` are written). */
+int mi355q_profile_durations(mi355q_context *ctx, double *kernel_us, size_t capacity,
+                             size_t *count, char *error, size_t error_capacity);
 
 /* Measured read bandwidth of HBM: one pass of 128-bit loads over a private
  * buffer of `bytes` (use >= 1 GiB to defeat the 256 MB memory-side cache),
