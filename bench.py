@@ -226,6 +226,11 @@ def bench_prefill(engine, ctx, args):
             "linears_per_step": 3,
             "algorithmic_flops_per_step": step_flops,
             "percent_of_f16_peak": round(100.0 * value / F16_MFMA_PEAK_TFLOPS, 2),
+            # what the matrix instruction sustains here from registers: alone, and with two or
+            # three packed-fp16 vector instructions per matrix instruction (in-register dequantization)
+            "measured_mfma_tflops": {"alone": round(ctx.probe_mfma_rate(0), 1),
+                                     "with_2_valu": round(ctx.probe_mfma_rate(2), 1),
+                                     "with_3_valu": round(ctx.probe_mfma_rate(3), 1)},
             "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
             **device_fields(ctx.info()),
         },

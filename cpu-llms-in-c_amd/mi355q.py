@@ -69,6 +69,7 @@ SIGNATURES = {
     "mi355q_profile_end": (_int, [_vp, _c.POINTER(_c.c_double), _c.POINTER(_u64), *_err]),
     "mi355q_profile_durations": (_int, [_vp, _vp, _sz, _c.POINTER(_sz), *_err]),
     "mi355q_probe_read_bandwidth": (_int, [_vp, _sz, _sz, _int, _int, _c.POINTER(_c.c_double), *_err]),
+    "mi355q_probe_mfma_rate": (_int, [_vp, _int, _int, _c.POINTER(_c.c_double), *_err]),
     "mi355q_q4_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32,
                                         _c.POINTER(_vp), *_err]),
     "mi355q_sym128_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _int, _u32, _c.POINTER(_vp), *_err]),
@@ -234,6 +235,11 @@ class Context:
         _call(self.lib.mi355q_probe_read_bandwidth, self.handle, nbytes, launch_bytes, repeats, variant,
               ctypes.byref(gbs))
         return gbs.value
+
+    def probe_mfma_rate(self, valu_per_mfma: int = 0, repeats: int = 3) -> float:
+        tflops = ctypes.c_double()
+        _call(self.lib.mi355q_probe_mfma_rate, self.handle, valu_per_mfma, repeats, ctypes.byref(tflops))
+        return tflops.value
 
     # ---- affine Q4 ----
     def q4_prepare(self, quants, meta_a, meta_b, N: int, K: int, meta_kind: int,

@@ -154,6 +154,15 @@ int mi355q_probe_read_bandwidth(mi355q_context *ctx, size_t bytes, size_t launch
                                 int repeats, int variant, double *gb_per_s,
                                 char *error, size_t error_capacity);
 
+/* Measured rate of the fp16 matrix instruction (v_mfma_f32_16x16x32_f16, fp32
+ * accumulation) with every SIMD issuing independent ones from registers and
+ * `valu_per_mfma` (0..4) packed-fp16 vector instructions between them — the mix of
+ * a GEMM that dequantizes weights in registers.  The figure to read a GEMM's
+ * TFLOP/s against, next to the datasheet's.  No counterpart in the reference (its
+ * targets have no matrix-instruction probe); same role as its bandwidth probes. */
+int mi355q_probe_mfma_rate(mi355q_context *ctx, int valu_per_mfma, int repeats,
+                           double *tflops, char *error, size_t error_capacity);
+
 /* ---- affine Q4, group 64: w[n][k] = scale[n][k/64] * q[n][k] + bias[n][k/64]
  *
  * quants: [N][K/64][32] bytes, element k of a row in byte k/2, even k in the

@@ -68,7 +68,7 @@ def test_small_shapes(engine, oracle, gpu, N, K, M, meta_kind):
 @pytest.mark.parametrize("M", [512, 2048])
 @pytest.mark.parametrize("N,K", [(17408, 5120), (5120, 17408)])
 def test_prefill_shapes(engine, oracle, gpu, N, K, M):
-    """BASELINE config 4: bf16 scale/bias, fp16 activations, fp16 output.  The oracle checks a
+    """Headline configuration 4 (27B MLP shapes at prefill row counts): bf16 scale/bias, fp16 activations, fp16 output.  The oracle checks a
     window of 48 output columns (every row of x) at full K; the rest of the output is checked for
     finiteness and, below, through linearity."""
     run_case(engine, oracle, gpu, N, K, M, engine.META_BF16_PLANES, engine.F16, engine.F16,

@@ -53,7 +53,7 @@ def run_case(engine, oracle, gpu, N, K, M, meta_kind, x_dtype, y_dtype, seed=7, 
 
 
 def test_config1_gemv_fp16(engine, oracle, gpu):
-    """BASELINE config 1: K=1024, N=3584, M=1, fp16 scale/bias, fp16 x, fp16 y."""
+    """Headline configuration 1 (the reference's own CPU-runnable case): K=1024, N=3584, M=1, fp16 scale/bias, fp16 x, fp16 y."""
     run_case(engine, oracle, gpu, 3584, 1024, 1, engine.META_F16_INTERLEAVED, engine.F16, engine.F16)
 
 
@@ -68,7 +68,7 @@ def test_edge_shapes(engine, oracle, gpu, N, K, M):
                                       ("gate_up", 17408, 5120), ("down", 5120, 17408)])
 @pytest.mark.parametrize("M", [1, 4, 8])
 def test_27b_layer_shapes(engine, oracle, gpu, name, N, K, M):
-    """BASELINE configs 2 and 3: bf16 scale/bias, fp16 activations, fp16 output."""
+    """Headline configurations 2 and 3 (27B layer shapes, decode and verify): bf16 scale/bias, fp16 activations, fp16 output."""
     run_case(engine, oracle, gpu, N, K, M, engine.META_BF16_PLANES, engine.F16, engine.F16,
              seed=11)
 

@@ -29,7 +29,7 @@ def check(engine, oracle, gpu, M, K, N, seed, bias=True):
 
 
 def test_config5(engine, oracle, gpu):
-    """BASELINE config 5: M=64, K=1024, N=4096."""
+    """Headline configuration 5 (SenseVoice encoder projection): M=64, K=1024, N=4096."""
     check(engine, oracle, gpu, 64, 1024, 4096, 31)
 
 
