@@ -63,6 +63,7 @@ LAYER = [  # name, N (output rows), K (input columns)
     ("down_proj", 5120, 17408),
 ]
 CONFIG1 = [("linear_0p8b", 3584, 1024)]
+LM_HEAD = [("lm_head", 248320, 5120)]  # the largest linear of the model: 698 MB, once per token
 PREFILL = [("gate_proj", 17408, 5120), ("up_proj", 17408, 5120), ("down_proj", 5120, 17408)]
 W8A8 = {"M": 64, "K": 1024, "N": 4096, "projections": 3}
 
@@ -351,7 +352,7 @@ def main():
     parser.add_argument("--copies", type=int, default=8)
     parser.add_argument("--rows", type=int, default=None,
                         help="activation rows M (default 1; 512 for --workload prefill)")
-    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "prefill", "w8a8"])
+    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "lm_head", "prefill", "w8a8"])
     parser.add_argument("--unfused", action="store_true",
                         help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
     parser.add_argument("--fused-mlp", action="store_true",
@@ -373,10 +374,12 @@ def main():
             args.steps, args.warmup = 100, 10
         with engine.Context(0) as ctx:  # raises without a GPU
             return (bench_prefill if args.workload == "prefill" else bench_w8a8)(engine, ctx, args)
-    shapes = LAYER if args.workload == "layer_m1" else CONFIG1
+    shapes = {"layer_m1": LAYER, "config1": CONFIG1, "lm_head": LM_HEAD}[args.workload]
     meta_kind = engine.META_BF16_PLANES if args.workload == "layer_m1" else engine.META_F16_INTERLEAVED
     M = args.rows
-    copies = args.copies if args.workload == "layer_m1" else max(args.copies, 600)
+    copies = {"layer_m1": args.copies, "config1": max(args.copies, 600), "lm_head": 2}[args.workload]
+    if args.workload == "lm_head" and args.steps == 400 and args.warmup == 40:
+        args.steps, args.warmup = 60, 6
     ctx = engine.Context(0)  # raises without a GPU
     info = ctx.info()
     calls, weights, host, x_ptr, y_ptr = build_workload(engine, ctx, shapes, M, copies, meta_kind,
@@ -416,8 +419,9 @@ def main():
     avg_kernel_us = kernel_ms * 1e3 / max(launches, 1)
     achieved = bytes_per_launch / (avg_kernel_us * 1e-6) / 1e9
     result = {
-        "metric": ("q4_gemv_hbm_gb_per_s_m%d_27b_layer" % M) if args.workload == "layer_m1"
-                  else "q4_gemv_hbm_gb_per_s_m%d_k1024_n3584" % M,
+        "metric": {"layer_m1": "q4_gemv_hbm_gb_per_s_m%d_27b_layer",
+                   "config1": "q4_gemv_hbm_gb_per_s_m%d_k1024_n3584",
+                   "lm_head": "q4_gemv_hbm_gb_per_s_m%d_lm_head_248320x5120"}[args.workload] % M,
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -433,7 +437,8 @@ def main():
         "config": {
             "workload": ("27B-shaped decoder layer linears q/k/v/o/gate/up/down at M=%d, affine-Q4 "
                          "g64, bf16 scale+bias, fp16 x and y" % M) if args.workload == "layer_m1"
-                        else "affine-Q4 g64 GEMV K=1024 N=3584 M=%d, fp16 scale+bias, fp16 x and y" % M,
+                        else "affine-Q4 g64 GEMV %s M=%d, fp16 scale+bias, fp16 x and y"
+                             % (" ".join("K=%d N=%d" % (K, N) for _, N, K in shapes), M),
             "linears_per_step": len(shapes),
             "launches_per_step": launches_per_step,
             "gate_up_silu_fused": bool(args.fused_mlp),

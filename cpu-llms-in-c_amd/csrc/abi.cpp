@@ -442,6 +442,57 @@ size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight)
     return weight ? weight->image_bytes : 0;
 }
 
+int mi355q_q4_dequant_rows(mi355q_context *ctx, const mi355q_q4_weight *weight, const uint32_t *rows,
+                           uint32_t count, void *out, int out_dtype, uint32_t flags, char *error,
+                           size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || rows == nullptr || out == nullptr || count == 0 ||
+        !dtype_valid(out_dtype)) {
+        set_error(error, error_capacity, "q4_dequant_rows: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "q4_dequant_rows: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    const bool rows_dev = flags & MI355Q_X_DEVICE, out_dev = flags & MI355Q_Y_DEVICE;
+    if ((flags & MI355Q_ASYNC) && !(rows_dev && out_dev)) {
+        set_error(error, error_capacity, "q4_dequant_rows: ASYNC needs device pointers throughout");
+        return MI355Q_ERROR_INVALID;
+    }
+    const Q4Device &dev = weight->dev;
+    if (!rows_dev)
+        for (uint32_t i = 0; i < count; ++i)
+            if (rows[i] >= dev.N) {
+                set_error(error, error_capacity, "q4_dequant_rows: row %u of a %u-row matrix", rows[i], dev.N);
+                return MI355Q_ERROR_INVALID;
+            }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t row_bytes = (size_t)count * sizeof(uint32_t);
+    const size_t out_bytes = (size_t)count * dev.K * dtype_bytes(out_dtype);
+    int status;
+    const uint32_t *rows_on_device = rows;
+    void *out_on_device = out;
+    if (!rows_dev) {
+        if ((status = ensure_stage(ctx, 0, row_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[0], rows, row_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "row id upload");
+        rows_on_device = (const uint32_t *)ctx->stage[0];
+    }
+    if (!out_dev) {
+        if ((status = ensure_stage(ctx, 1, out_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        out_on_device = ctx->stage[1];
+    }
+    hipError_t launched = q4_dequant_rows_launch(dev, rows_on_device, count, out_on_device, out_dtype,
+                                                 ctx->stream);
+    if (launched != hipSuccess) return fail_hip(launched, "q4 dequant rows launch", error, error_capacity);
+    if (!out_dev)
+        MI355Q_HIP(hipMemcpyAsync(out, out_on_device, out_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                   "row download");
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_dequant_rows sync");
+    return MI355Q_OK;
+}
+
 int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count,
                            const void *x, int x_dtype, uint32_t M, int y_dtype, int residual_dtype,
                            uint32_t flags, char *error, size_t error_capacity)

@@ -116,6 +116,9 @@ inline bool dtype_valid(int dtype) {
 hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
                             const uint16_t *meta_b, const Q4Device &dst,
                             hipStream_t stream);
+// rows of a prepared weight as plain numbers (device pointers)
+hipError_t q4_dequant_rows_launch(const Q4Device &w, const uint32_t *rows, uint32_t count, void *out,
+                                  int out_dtype, hipStream_t stream);
 // symmetric group-128 records -> affine group-64 planes (all device pointers)
 hipError_t sym128_to_affine_launch(const uint8_t *records, int output_blocked, uint32_t N,
                                    uint32_t K, uint8_t *quants, uint16_t *scales,

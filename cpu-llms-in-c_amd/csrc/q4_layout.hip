@@ -129,6 +129,62 @@ hipError_t sym128_to_affine_launch(const uint8_t *records, int output_blocked, u
     return hipGetLastError();
 }
 
+// Rows of the matrix as plain numbers, w[k] = fp32(scale) * q + fp32(bias) (multiply, then add:
+// no fused multiply-add), read back out of the stream tiles: the embedding lookup of
+// qwen38_q4_embedding_lookup (qwen38_global.metal:13-29).  One thread per eight columns.
+__global__ void __launch_bounds__(256)
+q4_dequant_rows_kernel(const uint4 *__restrict__ codes, const uint2 *__restrict__ meta, int meta_kind,
+                       uint32_t N, uint32_t K, uint32_t NT, const uint32_t *__restrict__ rows,
+                       uint32_t count, void *__restrict__ out, int out_dtype)
+{
+    const uint32_t words = K / 8u;
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (uint64_t)count * words) return;
+    const uint32_t item = (uint32_t)(index / words), word = (uint32_t)(index % words);
+    const uint32_t row = rows[item];
+    if (row >= N) return;  // as the reference kernel: an id past the table writes nothing
+    const uint32_t tile = row / kTileRows, r = row % kTileRows;
+    const uint32_t step = word / 16u, d = (word % 16u) / 4u, kq = word % 4u;
+    const uint64_t record = (uint64_t)step * NT + tile;
+    const uint4 packed = codes[record * 64u + kq * 16u + r];
+    const uint32_t bits = d == 0 ? packed.x : d == 1 ? packed.y : d == 2 ? packed.z : packed.w;
+    const uint2 pair = meta[record * 16u + r];
+    const uint32_t sb = (word % 16u) < 8u ? pair.x : pair.y;  // group 2*step or 2*step + 1
+    float scale, bias;
+    if (meta_kind == MI355Q_META_BF16_PLANES) {
+        scale = __builtin_bit_cast(float, sb << 16);
+        bias = __builtin_bit_cast(float, sb & 0xffff0000u);
+    } else {
+        scale = (float)__builtin_bit_cast(_Float16, (uint16_t)(sb & 0xffffu));
+        bias = (float)__builtin_bit_cast(_Float16, (uint16_t)(sb >> 16));
+    }
+#pragma unroll
+    for (uint32_t c = 0; c < 8u; ++c) {
+        // column c of the original code word: nibble c/2 of the low (even c) or high (odd c) half
+        const uint32_t q = (bits >> (16u * (c & 1u) + 4u * (c >> 1))) & 15u;
+        const float value = __fadd_rn(__fmul_rn(scale, (float)q), bias);
+        const size_t at = (size_t)item * K + 8u * word + c;
+        if (out_dtype == MI355Q_F32) {
+            ((float *)out)[at] = value;
+        } else if (out_dtype == MI355Q_F16) {
+            ((_Float16 *)out)[at] = (_Float16)value;
+        } else {
+            uint32_t raw = __builtin_bit_cast(uint32_t, value);
+            raw += 0x7fffu + ((raw >> 16) & 1u);
+            ((uint16_t *)out)[at] = (uint16_t)(raw >> 16);
+        }
+    }
+}
+
+hipError_t q4_dequant_rows_launch(const Q4Device &w, const uint32_t *rows, uint32_t count, void *out,
+                                  int out_dtype, hipStream_t stream)
+{
+    const uint64_t total = (uint64_t)count * (w.K / 8u);
+    hipLaunchKernelGGL(q4_dequant_rows_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0,
+                       stream, w.codes, w.meta, w.meta_kind, w.N, w.K, w.NT, rows, count, out, out_dtype);
+    return hipGetLastError();
+}
+
 hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,
                             const uint16_t *meta_b, const Q4Device &dst,
                             hipStream_t stream)

@@ -75,6 +75,7 @@ SIGNATURES = {
     "mi355q_sym128_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _int, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
+    "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_multi": (_int, [_vp, _c.POINTER(Q4Target), _u32, _vp, _int, _u32, _int, _int,
                                       _u32, *_err]),
@@ -255,6 +256,13 @@ class Context:
         _call(self.lib.mi355q_sym128_weight_prepare, self.handle, _ptr(records), N, K, record_order,
               flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
+
+    def q4_dequant_rows(self, weight: Q4Weight, rows, out_dtype: int = F32) -> np.ndarray:
+        rows = np.ascontiguousarray(rows, dtype=np.uint32)
+        out = np.empty((rows.size, weight.K), dtype=_NP_DTYPE[out_dtype])
+        _call(self.lib.mi355q_q4_dequant_rows, self.handle, weight.handle, _ptr(rows), rows.size, _ptr(out),
+              out_dtype, 0)
+        return out
 
     def q4_linear(self, weight: Q4Weight, x: np.ndarray, x_dtype: int, y_dtype: int = F32,
                   residual: np.ndarray | None = None, residual_dtype: int = F32,

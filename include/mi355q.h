@@ -197,6 +197,15 @@ void mi355q_q4_weight_destroy(mi355q_q4_weight *weight);
 /* Bytes of the original image this weight stands for: N*K/2 + N*(K/64)*4. */
 size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight);
 
+/* out[i][k] = scale * q + bias of row rows[i] (fp32 multiply then add, rounded once to
+ * out_dtype), [count][K]: the token-embedding lookup on a Q4 table,
+ * qwen38_q4_embedding_lookup (qwen38_global.metal:13-29).  MI355Q_X_DEVICE: `rows` is a
+ * device pointer (ids past the table then write nothing, as in the reference; host ids
+ * are checked and rejected with status 2); MI355Q_Y_DEVICE: `out` is a device pointer. */
+int mi355q_q4_dequant_rows(mi355q_context *ctx, const mi355q_q4_weight *weight,
+                           const uint32_t *rows, uint32_t count, void *out, int out_dtype,
+                           uint32_t flags, char *error, size_t error_capacity);
+
 /* y[m][n] = sum_k w[n][k] * x[m][k]  (+ residual[m][n] when residual != NULL)
  *
  * x: [M][K] of x_dtype (F16, F32 or BF16); y: [M][N] of y_dtype; residual:

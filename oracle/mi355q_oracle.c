@@ -178,6 +178,26 @@ static double q4_row_f64(const q4_matrix *w, size_t row, const void *x, int x_ki
     return total;
 }
 
+/* One dequantized row, fp32: w[k] = fp32(scale) * (float)q + fp32(bias), the expression
+ * of qwen38_q4_embedding_lookup (models/qwen3.8-27b/targets/apple-m3-pro/
+ * qwen38_global.metal:13-29) and of every CPU dot above, before any rounding of the
+ * result (the Metal kernel then rounds to half; callers do that with orc_f32_to_f16). */
+int orc_q4_dequantize_row(const uint8_t *quants, const void *meta_a, const void *meta_b,
+                          int meta_kind, uint32_t columns, uint32_t row, float *output)
+{
+    if (!quants || !meta_a || !output || columns == 0 || columns % 64u != 0) return 1;
+    q4_matrix w = {quants, (const uint16_t *)meta_a, (const uint16_t *)meta_b, meta_kind,
+                   columns / 64u};
+    for (size_t g = 0; g < w.groups; ++g) {
+        size_t block = (size_t)row * w.groups + g;
+        float scale, bias;
+        q4_group_meta(&w, block, &scale, &bias);
+        for (size_t j = 0; j < 64u; ++j)
+            output[g * 64u + j] = scale * (float)q4_code(&w, block, j) + bias;
+    }
+    return 0;
+}
+
 int orc_q4_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
                   int meta_kind, uint32_t N, uint32_t K,
                   const void *x, int x_kind, uint32_t M,

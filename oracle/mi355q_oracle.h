@@ -17,6 +17,9 @@
  *   orc_q4_dot_* / orc_q4_linear      numpy float64 brute force on unpacked
  *                                     codes; closed forms (all codes equal,
  *                                     zero scale, single hot nibble)
+ *   orc_q4_dequantize_row             numpy float32 arithmetic (no fused
+ *                                     multiply-add) on codes unpacked through
+ *                                     the uint32 view, fp16 and bf16 metadata
  *   orc_sym128_*                      the reference's own compiled q4_gemv /
  *                                     dequantize_q4_row (oracle/_ref), and
  *                                     the layout permutation its unit test
@@ -72,6 +75,8 @@ float orc_bf16_to_f32(uint16_t bits);
  * quants: [N][K/64][32] bytes; meta as per meta_kind (meta_b is NULL for the
  * interleaved kind).  x: [M][K] of x_kind.  y: [M][N] doubles (callers round).
  * rows [row_begin,row_end) are computed; threads <= 0 means the OpenMP default. */
+int orc_q4_dequantize_row(const uint8_t *quants, const void *meta_a, const void *meta_b,
+                          int meta_kind, uint32_t columns, uint32_t row, float *output);
 int orc_q4_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
                   int meta_kind, uint32_t N, uint32_t K,
                   const void *x, int x_kind, uint32_t M,

@@ -49,6 +49,8 @@ def lib() -> ctypes.CDLL:
         l.orc_q4_dot_f16x_seq.argtypes = [_vp, _vp, _vp, _sz, _sz]
         l.orc_q4_dot_f32x_seq.restype = _c.c_float
         l.orc_q4_dot_f32x_seq.argtypes = [_vp, _vp, _vp, _sz, _sz]
+        l.orc_q4_dequantize_row.restype = _int
+        l.orc_q4_dequantize_row.argtypes = [_vp, _vp, _vp, _int, _u32, _u32, _vp]
         l.orc_sym128_gemv.restype = None
         l.orc_sym128_gemv.argtypes = [_vp, _int, _u32, _u32, _vp, _vp, _int]
         l.orc_sym128_dequantize_row.restype = None
@@ -115,6 +117,17 @@ def q4_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_kind, M,
     if status != 0:
         raise ValueError(f"orc_q4_linear status {status}")
     return y
+
+
+def q4_dequantize_rows(quants, meta_a, meta_b, meta_kind, K, rows):
+    """fp32 [len(rows)][K]: scale * q + bias, unrounded."""
+    out = np.empty((len(rows), K), dtype=np.float32)
+    for i, row in enumerate(rows):
+        status = lib().orc_q4_dequantize_row(_p(quants), _p(meta_a), _p(meta_b), meta_kind, K, int(row),
+                                             _p(out[i]))
+        if status != 0:
+            raise ValueError(f"orc_q4_dequantize_row status {status}")
+    return out
 
 
 def sym128_gemv(records, output_blocked, rows, columns, x, threads=0):

@@ -194,3 +194,56 @@ def test_fused_gate_up_silu(engine, oracle, gpu, N, K, M, x_dtype):
     reference = g / (1.0 + np.exp(-g)) * u
     assert q4_relative_error(y, reference) <= TOLERANCE
     assert np.array_equal(y.view(np.uint32), queued.view(np.uint32))
+
+
+@pytest.mark.parametrize("meta_kind", ["META_F16_INTERLEAVED", "META_BF16_PLANES"])
+@pytest.mark.parametrize("N,K", [(1000, 5120), (33, 192)])
+def test_dequant_rows_embedding_lookup(engine, oracle, gpu, meta_kind, N, K):
+    """mi355q_q4_dequant_rows reads rows back out of the stream tiles: bit-exact with the oracle's
+    scale * q + bias in fp32, and with its fp16 / bf16 roundings (the reference's embedding kernel
+    writes half, qwen38_global.metal:13-29).  Ragged shapes exercise partial tiles and half steps."""
+    meta_kind = getattr(engine, meta_kind)
+    image = engine.synth_q4_affine(31, 0.02, N, K, meta_kind)
+    rows = np.array([0, N - 1, 17 % N, N // 2, 0], dtype=np.uint32)
+    weight = gpu.q4_prepare(*image, N, K, meta_kind)
+    try:
+        print(f"dequant rows N={N} K={K} meta={meta_kind}", flush=True)
+        as_f32 = gpu.q4_dequant_rows(weight, rows, engine.F32)
+        as_f16 = gpu.q4_dequant_rows(weight, rows, engine.F16)
+        as_bf16 = gpu.q4_dequant_rows(weight, rows, engine.BF16)
+        with pytest.raises(engine.Mi355qError) as info:
+            gpu.q4_dequant_rows(weight, [N], engine.F32)
+        assert info.value.status == engine.ERROR_INVALID
+    finally:
+        weight.destroy()
+    expect = oracle.q4_dequantize_rows(*image, meta_kind, K, rows)
+    assert np.array_equal(as_f32.view(np.uint32), expect.view(np.uint32))
+    assert np.array_equal(as_f16.view(np.uint16), expect.astype(np.float16).view(np.uint16))
+    assert np.array_equal(as_bf16, bf16_bits(expect).reshape(as_bf16.shape))
+
+
+def test_lm_head_sized_gemv(engine, oracle, gpu):
+    """The largest linear of the model, 248320 x 5120 (698 MB, qwen38_q4_lm_head,
+    qwen38_global.metal:39-61), fp16 activations and fp32 logits: three 48-row windows of the
+    output against the oracle, and the untouched logits between them against a second call
+    (bitwise repeatability)."""
+    N, K = 248320, 5120
+    rng = np.random.default_rng(5)
+    quants = rng.integers(0, 256, size=N * K // 2, dtype=np.uint8)
+    meta = np.empty(N * (K // 64) * 2, dtype=np.uint16)
+    meta[0::2] = (rng.random(N * (K // 64), dtype=np.float32) * 0.01 + 0.001).astype(np.float16).view(np.uint16)
+    meta[1::2] = (rng.standard_normal(N * (K // 64), dtype=np.float32) * 0.05).astype(np.float16).view(np.uint16)
+    x = make_x(engine, 3, 1, K, engine.F16)
+    weight = gpu.q4_prepare(quants, meta, None, N, K, engine.META_F16_INTERLEAVED)
+    try:
+        print("lm head case", flush=True)
+        y = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+        again = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+    finally:
+        weight.destroy()
+    assert np.array_equal(y.view(np.uint32), again.view(np.uint32))
+    assert np.all(np.isfinite(y))
+    for begin in (0, 124111, N - 48):
+        ref = oracle.q4_linear(quants, meta, None, engine.META_F16_INTERLEAVED, N, K, x, engine.F16, 1,
+                               rows=(begin, begin + 48))[:, begin:begin + 48]
+        assert q4_relative_error(y[:, begin:begin + 48], ref) <= TOLERANCE

@@ -189,3 +189,26 @@ def test_qwen38_synthetic_recipe_and_bf16_weight_flavour(oracle):
     got_b = oracle.q4_linear(quants, s, b, 1, N, K, xb, oracle.X_BF16, 1,
                              weight_rounding=oracle.W_ROUND_BF16)
     assert np.allclose(got_b, expect_b, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("meta_kind", [0, 1])
+def test_dequantize_row_equals_numpy_float32(oracle, meta_kind):
+    """orc_q4_dequantize_row (qwen38_global.metal:13-29) against numpy float32 arithmetic — a
+    rounded multiply, then a rounded add, numpy never fuses them — on codes unpacked through the
+    uint32 view; a wrong nibble, byte, group or plane index changes some element."""
+    rng = np.random.default_rng(11)
+    N, K = 23, 448
+    quants, meta_a, meta_b = random_image(rng, N, K, meta_kind)
+    codes = unpack_codes(quants, N, K).astype(np.float32)
+    if meta_kind == 0:
+        meta = np.asarray(meta_a).reshape(N, K // 64, 2)
+        scale = meta[..., 0].copy().view(np.float16).astype(np.float32)
+        bias = meta[..., 1].copy().view(np.float16).astype(np.float32)
+    else:
+        scale = bf16_to_f32(meta_a).reshape(N, K // 64)
+        bias = bf16_to_f32(meta_b).reshape(N, K // 64)
+    expect = np.repeat(scale, 64, axis=1) * codes + np.repeat(bias, 64, axis=1)
+    assert expect.dtype == np.float32
+    rows = [0, 7, 22, 7]
+    got = oracle.q4_dequantize_rows(quants, meta_a, meta_b, meta_kind, K, rows)
+    assert np.array_equal(got.view(np.uint32), expect[rows].view(np.uint32))
