@@ -124,10 +124,18 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         const uint32_t count = wave < span ? (span - wave + W - 1u) / W : 0u;
         const uint32_t step0 = first + wave;
 
-        // Loads are issued unconditionally (the step index is clamped instead),
-        // so the number in flight is known at compile time and each step waits
-        // only for its own data.
+        // In the main loop every step refills the slot it consumed, unconditionally, so
+        // the number of loads in flight is known at compile time and each step waits only
+        // for its own data; only the first D loads (a wave may own fewer steps) clamp.
         auto issue = [&](uint32_t i, StepData<TB> &slot) {
+            const uint32_t step = step0 + i * W;
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) {
+                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * NT * 64u);
+                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * NT * 16u);
+            }
+        };
+        auto issue_clamped = [&](uint32_t i, StepData<TB> &slot) {
             const uint32_t clamped = i < count ? i : (count ? count - 1u : 0u);
             uint32_t step = step0 + clamped * W;
             step = step < p.T ? step : p.T - 1u;
@@ -163,7 +171,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 
         StepData<TB> ring[D];
 #pragma unroll
-        for (int u = 0; u < D; ++u) issue(u, ring[u]);
+        for (int u = 0; u < D; ++u) issue_clamped(u, ring[u]);
 
         if (first > slice_begin) __syncthreads();  // everyone is done with the previous chunk
 #pragma unroll
@@ -176,48 +184,63 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         }
         __syncthreads();
 
-        for (uint32_t base = 0; base < count; base += D) {
+        auto consume = [&](uint32_t i, const StepData<TB> &slot) {
+            const uint4 *xp = xs_lane + (size_t)(wave + i * W) * 16u * MP;
+            const half8 a0 = __builtin_bit_cast(half8, xp[0]);
+            const half8 a1 = __builtin_bit_cast(half8, xp[4 * MP]);
+            const half8 a2 = __builtin_bit_cast(half8, xp[8 * MP]);
+            const half8 a3 = __builtin_bit_cast(half8, xp[12 * MP]);
+
+            // per-group activation sums, laid out like the products (row 4*kq+j)
+            floatx4 xs0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ones, zero, 0, 0, 0);
+            xs0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ones, xs0, 0, 0, 0);
+            floatx4 xs1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, ones, zero, 0, 0, 0);
+            xs1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, ones, xs1, 0, 0, 0);
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) {
+                const uint4 q = slot.q[tb];
+                const uint2 m = slot.m[tb];
+                float scale, bias;
+                floatx4 c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, unpack8(q.x, masks), zero,
+                                                                   0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, unpack8(q.y, masks), c, 0, 0, 0);
+                decode_meta(m.x, BF, scale, bias);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    acc[tb][j] = __builtin_fmaf(scale, c[j], acc[tb][j]);
+                    acc[tb][j] = __builtin_fmaf(bias, xs0[j], acc[tb][j]);
+                }
+                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, unpack8(q.z, masks), zero, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, unpack8(q.w, masks), c, 0, 0, 0);
+                decode_meta(m.y, BF, scale, bias);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    acc[tb][j] = __builtin_fmaf(scale, c[j], acc[tb][j]);
+                    acc[tb][j] = __builtin_fmaf(bias, xs1[j], acc[tb][j]);
+                }
+            }
+        };
+        // main part: whole groups of D steps whose refills all exist
+        const uint32_t main_end = count > (uint32_t)D ? (count - D) / D * D : 0u;
+        for (uint32_t base = 0; base < main_end; base += D) {
 #pragma unroll
             for (int u = 0; u < D; ++u) {
-                const uint32_t i = base + u;
-                if (i >= count) break;
-                const uint4 *xp = xs_lane + (size_t)(wave + i * W) * 16u * MP;
-                const half8 a0 = __builtin_bit_cast(half8, xp[0]);
-                const half8 a1 = __builtin_bit_cast(half8, xp[4 * MP]);
-                const half8 a2 = __builtin_bit_cast(half8, xp[8 * MP]);
-                const half8 a3 = __builtin_bit_cast(half8, xp[12 * MP]);
-
-                // per-group activation sums, laid out like the products (row 4*kq+j)
-                floatx4 xs0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ones, zero, 0, 0, 0);
-                xs0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ones, xs0, 0, 0, 0);
-                floatx4 xs1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, ones, zero, 0, 0, 0);
-                xs1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, ones, xs1, 0, 0, 0);
-#pragma unroll
-                for (int tb = 0; tb < TB; ++tb) {
-                    const uint4 q = ring[u].q[tb];
-                    const uint2 m = ring[u].m[tb];
-                    float scale, bias;
-                    floatx4 c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, unpack8(q.x, masks), zero,
-                                                                       0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, unpack8(q.y, masks), c, 0, 0, 0);
-                    decode_meta(m.x, BF, scale, bias);
-#pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
-                        acc[tb][j] = __builtin_fmaf(scale, c[j], acc[tb][j]);
-                        acc[tb][j] = __builtin_fmaf(bias, xs0[j], acc[tb][j]);
-                    }
-                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, unpack8(q.z, masks), zero, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, unpack8(q.w, masks), c, 0, 0, 0);
-                    decode_meta(m.y, BF, scale, bias);
-#pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
-                        acc[tb][j] = __builtin_fmaf(scale, c[j], acc[tb][j]);
-                        acc[tb][j] = __builtin_fmaf(bias, xs1[j], acc[tb][j]);
-                    }
-                }
-                issue(i + D, ring[u]);  // refill the slot just consumed
+                consume(base + u, ring[u]);
+                issue(base + u + D, ring[u]);  // refill the slot just consumed
             }
         }
+        // the last (at most 2D - 1) steps: refill only while steps remain, then drain
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const uint32_t i = main_end + u;
+            if (i < count) {
+                consume(i, ring[u]);
+                if (i + D < count) issue(i + D, ring[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < D; ++u)
+            if (main_end + D + u < count) consume(main_end + D + u, ring[u]);
     }
 
     // ---- add the waves' partial sums in wave order, then store
