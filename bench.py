@@ -355,6 +355,9 @@ def main():
     parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "lm_head", "prefill", "w8a8"])
     parser.add_argument("--unfused", action="store_true",
                         help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
+    parser.add_argument("--graph", action="store_true",
+                        help="replay each step from a recorded HIP graph (one host call per step) in "
+                             "the timed pass; the per-kernel pass stays eager")
     parser.add_argument("--fused-mlp", action="store_true",
                         help="gate|up launch applies silu(gate)*up (one output instead of two)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -392,11 +395,19 @@ def main():
         for step in range(count):
             ctx.q4_sequence(calls[step % copies])
 
-    run_steps(args.warmup)
+    graphs = [ctx.q4_sequence_record(c) for c in calls] if args.graph else None
+
+    def run_timed(count):
+        if graphs is None:
+            return run_steps(count)
+        for step in range(count):
+            ctx.graph_launch(graphs[step % copies])
+
+    run_timed(args.warmup)
     ctx.sync()
     t0 = time.perf_counter()
     ctx.timer_begin()
-    run_steps(args.steps)
+    run_timed(args.steps)
     gpu_ms = ctx.timer_end()  # waits for the stream
     ctx.sync()
     wall = time.perf_counter() - t0
@@ -442,6 +453,7 @@ def main():
             "linears_per_step": len(shapes),
             "launches_per_step": launches_per_step,
             "gate_up_silu_fused": bool(args.fused_mlp),
+            "steps_replayed_from_graph": bool(args.graph),
             "algorithmic_bytes_per_step": step_bytes,
             "weight_copies_rotated": copies,
             "rotated_bytes": step_bytes * copies,
@@ -474,6 +486,8 @@ def main():
         import oracle  # test infrastructure, used here only as the timed CPU baseline
         result["cpu_baseline"] = cpu_baseline(oracle, shapes, host, M, meta_kind)
     print(json.dumps(result), flush=True)
+    for graph in graphs or []:
+        ctx.graph_destroy(graph)
     for copy in weights:
         for weight in copy:
             weight.destroy()

@@ -28,6 +28,11 @@ int ensure_stage(mi355q_context *ctx, int slot, size_t bytes, char *error,
                  size_t error_capacity)
 {
     if (bytes <= ctx->stage_bytes[slot]) return MI355Q_OK;
+    if (ctx->capturing) {  // no allocation while a graph is being recorded
+        set_error(error, error_capacity, "staging buffer %d would grow during graph capture", slot);
+        return MI355Q_ERROR_RUNTIME;
+    }
+    ctx->stage_generation += 1;
     MI355Q_HIP(hipStreamSynchronize(ctx->stream), "sync before staging growth");
     if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
     ctx->stage[slot] = nullptr;
@@ -651,6 +656,93 @@ int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, 
         }
     }
     return MI355Q_OK;
+}
+
+// ---- recorded sequences ---------------------------------------------------------
+
+struct mi355q_graph {
+    mi355q_context *ctx;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    uint64_t stage_generation;
+};
+
+int mi355q_q4_sequence_record(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,
+                              mi355q_graph **out, char *error, size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    if (ctx == nullptr || out == nullptr || calls == nullptr || count == 0) {
+        set_error(error, error_capacity, "q4_sequence_record: null argument or no calls");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (ctx->profiling || ctx->capturing) {
+        set_error(error, error_capacity, "q4_sequence_record: not while profiling or recording");
+        return MI355Q_ERROR_INVALID;
+    }
+    // once for real: checks every argument and sizes the internal staging buffers, so that
+    // the recording itself allocates nothing
+    int status = mi355q_q4_linear_sequence(ctx, calls, count, error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+
+    mi355q_graph *recorded = new (std::nothrow) mi355q_graph();
+    if (recorded == nullptr) {
+        set_error(error, error_capacity, "q4_sequence_record: out of host memory");
+        return MI355Q_ERROR_RUNTIME;
+    }
+    recorded->ctx = ctx;
+    recorded->graph = nullptr;
+    recorded->exec = nullptr;
+    recorded->stage_generation = ctx->stage_generation;
+    hipError_t hip = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (hip != hipSuccess) {
+        delete recorded;
+        return fail_hip(hip, "hipStreamBeginCapture", error, error_capacity);
+    }
+    ctx->capturing = true;
+    status = mi355q_q4_linear_sequence(ctx, calls, count, error, error_capacity);
+    ctx->capturing = false;
+    hip = hipStreamEndCapture(ctx->stream, &recorded->graph);  // always ends the capture
+    if (status == MI355Q_OK && hip != hipSuccess)
+        status = fail_hip(hip, "hipStreamEndCapture", error, error_capacity);
+    if (status == MI355Q_OK) {
+        hip = hipGraphInstantiate(&recorded->exec, recorded->graph, nullptr, nullptr, 0);
+        if (hip != hipSuccess) status = fail_hip(hip, "hipGraphInstantiate", error, error_capacity);
+    }
+    if (status != MI355Q_OK) {
+        mi355q_graph_destroy(recorded);
+        return status;
+    }
+    *out = recorded;
+    return MI355Q_OK;
+}
+
+int mi355q_graph_launch(mi355q_context *ctx, mi355q_graph *graph, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || graph == nullptr || graph->ctx != ctx) {
+        set_error(error, error_capacity, "graph_launch: null argument or another context's graph");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (graph->stage_generation != ctx->stage_generation) {
+        set_error(error, error_capacity,
+                  "graph_launch: the context reallocated a staging buffer since this sequence was "
+                  "recorded; record it again");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (ctx->profiling) {
+        set_error(error, error_capacity, "graph_launch: per-kernel profiling does not see recorded kernels");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipGraphLaunch(graph->exec, ctx->stream), "hipGraphLaunch");
+    return MI355Q_OK;
+}
+
+void mi355q_graph_destroy(mi355q_graph *graph)
+{
+    if (graph == nullptr) return;
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
 }
 
 }  // extern "C"

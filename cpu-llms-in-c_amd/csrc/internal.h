@@ -61,6 +61,10 @@ struct mi355q_context {
     // 4 fp32 partial sums of a K-split GEMM
     void *stage[5];
     size_t stage_bytes[5];
+    // bumped whenever a staging buffer is reallocated: recorded graphs hold the old
+    // pointers and refuse to run once this has moved on
+    uint64_t stage_generation;
+    bool capturing;  // between hipStreamBeginCapture and EndCapture on `stream`
 };
 
 struct mi355q_q4_weight {

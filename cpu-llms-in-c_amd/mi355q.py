@@ -84,6 +84,9 @@ SIGNATURES = {
     "mi355q_hook_q4_gemv": (_int, [_vp, _int, _sz, _sz, _vp, _vp]),
     "mi355q_hook_last_error": (_int, [_c.c_char_p, _sz]),
     "mi355q_hook_release": (None, []),
+    "mi355q_q4_sequence_record": (_int, [_vp, _c.POINTER(Q4Call), _sz, _c.POINTER(_vp), *_err]),
+    "mi355q_graph_launch": (_int, [_vp, _vp, *_err]),
+    "mi355q_graph_destroy": (None, [_vp]),
     "mi355q_w8a8_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_w8a8_weight_destroy": (None, [_vp]),
     "mi355q_quantize_i8": (_int, [_vp, _vp, _u32, _u32, _vp, _vp, _u32, *_err]),
@@ -344,6 +347,18 @@ class Context:
                            acc_ptr=None, asynchronous: bool = True):
         _call(self.lib.mi355q_w8a8_linear, self.handle, weight, q_ptr, scales_ptr, M, bias_ptr, out_ptr,
               acc_ptr, X_DEVICE | Y_DEVICE | (ASYNC if asynchronous else 0))
+
+    def q4_sequence_record(self, calls):
+        """Records the calls into a graph (running them once); returns the graph handle."""
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_q4_sequence_record, self.handle, calls, len(calls), ctypes.byref(out))
+        return out
+
+    def graph_launch(self, graph):
+        _call(self.lib.mi355q_graph_launch, self.handle, graph)
+
+    def graph_destroy(self, graph):
+        self.lib.mi355q_graph_destroy(graph)
 
     def q4_sequence(self, calls):
         """calls: a ctypes array of Q4Call (build once, reuse)."""

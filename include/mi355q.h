@@ -32,6 +32,7 @@ extern "C" {
 
 typedef struct mi355q_context mi355q_context;
 typedef struct mi355q_q4_weight mi355q_q4_weight;
+typedef struct mi355q_graph mi355q_graph;
 typedef struct mi355q_w8a8_weight mi355q_w8a8_weight;
 
 enum {
@@ -256,6 +257,20 @@ typedef struct {
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls,
                               size_t count, char *error, size_t error_capacity);
+
+/* The same run of calls recorded once into a HIP graph and replayed with one host call
+ * per run: for loops whose kernels are shorter than the host's per-launch cost (a small
+ * model's decode step).  Recording executes the calls once (which also sizes the
+ * library's staging buffers), then captures them; replays use the recorded pointers and
+ * shapes.  A replay is asynchronous on the context's stream.  If a later call makes the
+ * context grow a staging buffer, recorded graphs refuse to launch (status 2): record
+ * again.  The counterpart of the reference committing one pre-encoded command buffer per
+ * token (qwen38_m3_decode.m:1614-1716). */
+int mi355q_q4_sequence_record(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,
+                              mi355q_graph **out, char *error, size_t error_capacity);
+int mi355q_graph_launch(mi355q_context *ctx, mi355q_graph *graph,
+                        char *error, size_t error_capacity);
+void mi355q_graph_destroy(mi355q_graph *graph);
 
 /* ---- drop-ins with the reference's own hook signatures ----------------------
  *

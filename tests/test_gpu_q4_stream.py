@@ -247,3 +247,63 @@ def test_lm_head_sized_gemv(engine, oracle, gpu):
         ref = oracle.q4_linear(quants, meta, None, engine.META_F16_INTERLEAVED, N, K, x, engine.F16, 1,
                                rows=(begin, begin + 48))[:, begin:begin + 48]
         assert q4_relative_error(y[:, begin:begin + 48], ref) <= TOLERANCE
+
+
+def test_recorded_sequence_replays(engine, oracle, gpu):
+    """mi355q_q4_sequence_record / mi355q_graph_launch: three calls (shared-x pair at M=1, an fp32
+    activation that goes through the conversion kernel, an M=8 call that is cut in K slices and
+    reduced) recorded into one graph; every replay, with eager work and synchronisation in between
+    and fresh inputs, must equal the eager sequence bit for bit.  A graph is refused once the
+    context has reallocated a staging buffer."""
+    K1, N1, K2, N2 = 1536, 640, 8704, 320
+    images = [engine.synth_q4_affine(80 + i, 0.02, n, k, engine.META_BF16_PLANES)
+              for i, (n, k) in enumerate([(N1, K1), (N1, K1), (N2, K2), (N2, K2)])]
+    weights = [gpu.q4_prepare(*image, n, k, engine.META_BF16_PLANES)
+               for image, (n, k) in zip(images, [(N1, K1), (N1, K1), (N2, K2), (N2, K2)])]
+    pointers, graph = [], None
+    try:
+        x1 = make_x(engine, 1, 1, K1, engine.F16)
+        x2 = make_x(engine, 2, 2, K2, engine.F32)
+        x3 = make_x(engine, 3, 8, K2, engine.F16)
+        x_ptr = [gpu.to_device(x) for x in (x1, x2, x3)]
+        y_shapes = [(1, N1), (1, N1), (2, N2), (8, N2)]
+        y_ptr = [gpu.alloc(m * n * 4) for m, n in y_shapes]
+        pointers = x_ptr + y_ptr
+        calls = engine.make_calls([
+            ([(weights[0], y_ptr[0]), (weights[1], y_ptr[1])], x_ptr[0], engine.F16, 1, engine.F32),
+            ((weights[2], y_ptr[2]), x_ptr[1], engine.F32, 2, engine.F32),
+            ((weights[3], y_ptr[3]), x_ptr[2], engine.F16, 8, engine.F32)])
+
+        def outputs():
+            gpu.sync()
+            return [gpu.download(p, shape, np.float32) for p, shape in zip(y_ptr, y_shapes)]
+
+        print("recorded sequence case", flush=True)
+        graph = gpu.q4_sequence_record(calls)
+        for replay in range(3):
+            # new activations, an eager run as the expectation, outputs wiped, then the replay
+            for pointer, x, seed in zip(x_ptr, (x1, x2, x3), (11, 12, 13)):
+                gpu.upload(pointer, make_x(engine, seed + 10 * replay, x.shape[0], x.shape[1],
+                                           engine.F32 if x.dtype == np.float32 else engine.F16))
+            gpu.q4_sequence(calls)
+            expect = outputs()
+            for pointer, shape in zip(y_ptr, y_shapes):
+                gpu.upload(pointer, np.zeros(shape, dtype=np.float32))
+            gpu.graph_launch(graph)
+            got = outputs()
+            for a, b in zip(got, expect):
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), f"replay {replay}"
+            assert all(np.any(a != 0) for a in got)
+        # a host-pointer call larger than any before it grows a staging buffer: the graph is stale
+        big = gpu.q4_linear(weights[3], make_x(engine, 5, 16, K2, engine.F16), engine.F16, engine.F32)
+        assert big.shape == (16, N2)
+        with pytest.raises(engine.Mi355qError) as info:
+            gpu.graph_launch(graph)
+        assert info.value.status == engine.ERROR_INVALID
+    finally:
+        if graph is not None:
+            gpu.graph_destroy(graph)
+        for pointer in pointers:
+            gpu.free(pointer)
+        for w in weights:
+            w.destroy()
