@@ -336,7 +336,6 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     constexpr int NTX = NTW + (XT ? 1 : 0);
     constexpr int XI = MI / 4;  // row fragments of the shared tile per wave
     typedef __attribute__((address_space(3))) void *lds_ptr;
-    typedef const __attribute__((address_space(1))) void *global_ptr;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -360,6 +359,9 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         m = m < p.M ? m : p.M - 1u;
         a_source[j] = p.x + (size_t)m * p.K + 8u * (r ^ (local & 15u));
     }
+    // The copies into LDS are asm: the compiler would otherwise make every wave drain all of
+    // its outstanding loads before the first LDS read behind the barrier, the weights it
+    // prefetched two steps ahead included.  The wait before the barrier counts them instead.
     auto fetch_a = [&](uint32_t step, int buffer) {
 #pragma unroll
         for (int j = 0; j < AJ; ++j) {
@@ -367,8 +369,12 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
             const uint32_t octet = r ^ (((BM / 4) * wave + 4u * j + kq) & 15u);
             const _Float16 *source = a_source[j] + k;
             if (k + 8u * octet >= p.K) source -= 64;
-            __builtin_amdgcn_global_load_lds((global_ptr)source,
-                                             (lds_ptr)&a_lds[buffer][(BM / 4) * wave + 4u * j][0], 16, 0, 0);
+            const uint32_t lds_base =
+                (uint32_t)(uintptr_t)(lds_ptr)&a_lds[buffer][(BM / 4) * wave + 4u * j][0];
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :
+                         : "v"(source), "s"(lds_base)
+                         : "memory");
         }
     };
     auto fetch_tile = [&](uint32_t step, uint32_t tile, uint4 &codes, uint2 &meta) {
@@ -405,8 +411,10 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     // instructions and the LDS read that follow it in the source to that slot.
     const uint32_t last_step = step_end - 1u;
     auto clamp_step = [&](uint32_t step) { return step < last_step ? step : last_step; };
-    uint4 b_codes[NTX], next_codes[NTX];
-    uint2 b_meta[NTX], next_meta[NTX];
+    // three register sets of codes and metadata, in rotation: the step being multiplied, the
+    // next one, and the one after that still in flight (weights come from HBM: two steps of lead)
+    uint4 b_codes[3][NTX];
+    uint2 b_meta[3][NTX];
     half2v b_frag[2][NTX][4];  // [set][tile][column pair group]: 8 weights of a lane
     half8 a_frag[MI];
     half8 a_shared[XI];
@@ -458,11 +466,12 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     };
 
     fetch_a(step_begin, 0);
-    fetch_b(step_begin, b_codes, b_meta);
+    fetch_b(step_begin, b_codes[0], b_meta[0]);
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     fetch_a(clamp_step(step_begin + 1u), 1);
-    fetch_b(clamp_step(step_begin + 1u), next_codes, next_meta);
+    fetch_b(clamp_step(step_begin + 1u), b_codes[1], b_meta[1]);
+    fetch_b(clamp_step(step_begin + 2u), b_codes[2], b_meta[2]);
 #pragma unroll
     for (int i = 0; i < MI; ++i) a_frag[i] = read_frag(0, 0, i);
     if (XT) {
@@ -471,35 +480,46 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     }
     static_for<PIECES>([&](auto piece_c) {
         static_for<3>([&](auto stage_c) {
-            dequant_stage<decltype(stage_c)::value, decltype(piece_c)::value, 0>(b_codes, b_meta, masks,
+            dequant_stage<decltype(stage_c)::value, decltype(piece_c)::value, 0>(b_codes[0], b_meta[0], masks,
                                                                                   merged, centred, b_frag[0]);
             asm volatile("s_nop 1");  // packed-fp16 result to its reader: one wait state
         });
     });
 
-    for (uint32_t step = step_begin; step < step_end; ++step) {
+    // One step with the register set `cur` (this step's weights) and `next` (the next step's);
+    // `cur` is free after quarter 2 and receives the weights of step + 3.
+    auto one_step = [&](uint32_t step, auto cur_c, auto next_c) {
+        constexpr int cur = decltype(cur_c)::value, next = decltype(next_c)::value;
         const int buffer = (int)((step - step_begin) & 1u);
         static_for<3>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
             __builtin_amdgcn_sched_barrier(0);
             quarter(std::integral_constant<int, (d & 1)>(), std::integral_constant<int, d + 1>(), buffer,
-                    b_codes, b_meta);
+                    b_codes[cur], b_meta[cur]);
         });
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): fetches landed, LDS reads done
+        // everything but the newest weight fetch (2 * NTX loads, of step + 2) has landed: the
+        // activations and weights of step + 1; and this wave's LDS reads are done
+        __builtin_amdgcn_s_waitcnt(0x0070 | (2 * NTX));
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         fetch_a(clamp_step(step + 2u), buffer);
-        quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), buffer ^ 1, next_codes,
-                next_meta);
+        quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), buffer ^ 1, b_codes[next],
+                b_meta[next]);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < NTX; ++t) {
-            b_codes[t] = next_codes[t];
-            b_meta[t] = next_meta[t];
-        }
-        fetch_b(clamp_step(step + 2u), next_codes, next_meta);
+        fetch_b(clamp_step(step + 3u), b_codes[cur], b_meta[cur]);
+    };
+    // whole rotations in a loop without branches (the compiler then counts the loads in flight
+    // exactly), the last one or two steps after it
+    uint32_t step = step_begin;
+    for (; step + 3u <= step_end; step += 3u) {
+        one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
+        one_step(step + 1u, std::integral_constant<int, 1>(), std::integral_constant<int, 2>());
+        one_step(step + 2u, std::integral_constant<int, 2>(), std::integral_constant<int, 0>());
     }
+    if (step < step_end) one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
+    if (step + 1u < step_end)
+        one_step(step + 1u, std::integral_constant<int, 1>(), std::integral_constant<int, 2>());
 
     __builtin_amdgcn_s_waitcnt(0x0f70);  // the last step's spare fetch into LDS has landed
 
