@@ -611,8 +611,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     // The choice minimises a microsecond estimate fitted to sweeps over every variant
     // and split on this GPU: a workgroup that has a compute unit to itself sustains
     // `alone` of the matrix-instruction peak, co-resident workgroups `shared` together;
-    // a grid beyond one resident set pays ~0.3 of a workgroup time for its ragged
-    // end, and a K split pays for its fp32 partials at ~5 TB/s.
+    // a grid that is not a whole number of resident sets pays ~0.3 of a workgroup time for
+    // its ragged end, and a K split pays for its fp32 partials at ~4.3 TB/s.
     struct Variant {
         int bm, ntw, extra;
         int resident;          // workgroups that fit one compute unit (registers, LDS)
@@ -620,10 +620,10 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     };
     // 0-5: two workgroups per compute unit overlap each other; 6, 7: the pipelined kernel,
     // one workgroup per compute unit
-    static const Variant variants[] = {{128, 4, 0, 2, 0.407, 0.495}, {128, 2, 0, 2, 0.346, 0.451},
-                                       {64, 4, 0, 3, 0.354, 0.464},  {64, 4, 1, 2, 0.384, 0.478},
-                                       {64, 2, 0, 4, 0.350, 0.428},  {64, 2, 1, 2, 0.399, 0.469},
-                                       {128, 4, 0, 1, 0.449, 0.360}, {128, 4, 1, 1, 0.429, 0.373}};
+    static const Variant variants[] = {{128, 4, 0, 2, 0.412, 0.502}, {128, 2, 0, 2, 0.350, 0.463},
+                                       {64, 4, 0, 3, 0.358, 0.478},  {64, 4, 1, 2, 0.385, 0.470},
+                                       {64, 2, 0, 4, 0.350, 0.443},  {64, 2, 1, 2, 0.399, 0.473},
+                                       {128, 4, 0, 1, 0.476, 0.450}, {128, 4, 1, 1, 0.445, 0.430}};
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     int best = 0;
     uint32_t best_splits = 1;
@@ -646,12 +646,16 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             double cost;
             if (groups <= cus)
                 cost = peak_us / c.alone;
-            else if (groups <= slots)
-                cost = (double)((groups + cus - 1) / cus) * peak_us / c.shared;
+            else if (groups <= slots) {
+                // k of the `resident` workgroups a compute unit could hold: in between
+                const double k = (double)((groups + cus - 1) / cus);
+                const double sustained = c.alone + (c.shared - c.alone) * (k - 1.0) / (c.resident - 1.0);
+                cost = k * peak_us / sustained;
+            }
             else
-                cost = ((double)groups / slots + 0.315) * c.resident * peak_us / c.shared;
+                cost = ((double)groups / slots + (groups % slots ? 0.29 : 0.0)) * c.resident * peak_us / c.shared;
             if (splits > 1)  // fp32 partials written and read back
-                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.5e12 * 1.0e6;
+                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.3e12 * 1.0e6;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;

@@ -254,7 +254,9 @@ def test_recorded_sequence_replays(engine, oracle, gpu):
     activation that goes through the conversion kernel, an M=8 call that is cut in K slices and
     reduced) recorded into one graph; every replay, with eager work and synchronisation in between
     and fresh inputs, must equal the eager sequence bit for bit.  A graph is refused once the
-    context has reallocated a staging buffer."""
+    context has reallocated a staging buffer (a context of its own, so that what other tests did
+    to the shared one does not decide whether the last call grows a buffer)."""
+    gpu = engine.Context(0)  # the fixture only decides whether the test runs at all
     K1, N1, K2, N2 = 1536, 640, 8704, 320
     images = [engine.synth_q4_affine(80 + i, 0.02, n, k, engine.META_BF16_PLANES)
               for i, (n, k) in enumerate([(N1, K1), (N1, K1), (N2, K2), (N2, K2)])]
@@ -307,3 +309,4 @@ def test_recorded_sequence_replays(engine, oracle, gpu):
             gpu.free(pointer)
         for w in weights:
             w.destroy()
+        gpu.close()
