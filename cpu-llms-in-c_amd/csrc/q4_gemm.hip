@@ -349,39 +349,38 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
     if (step_begin >= step_end) return;  // uniform over the workgroup
 
-    // Rows beyond M re-read the last row and columns beyond K re-read the previous group
-    // (finite values against zero weights): both stay in bounds and never reach y.
-    const _Float16 *a_source[AJ];
+    // Activation stage.  The host sends only whole 128-column steps (K % 128 == 0) and
+    // M * K * 2 < 4 GiB here, so a lane's piece of the stage is one scalar base (advancing 256
+    // bytes per step) plus a 32-bit byte offset fixed for the whole kernel.  Rows beyond M
+    // re-read the last row: they stay in bounds and never reach y.
+    uint32_t a_offset[AJ];
 #pragma unroll
     for (int j = 0; j < AJ; ++j) {
         const uint32_t local = (BM / 4) * wave + 4u * j + kq;
         uint32_t m = m0 + local;
         m = m < p.M ? m : p.M - 1u;
-        a_source[j] = p.x + (size_t)m * p.K + 8u * (r ^ (local & 15u));
+        a_offset[j] = (m * p.K + 8u * (r ^ (local & 15u))) * (uint32_t)sizeof(_Float16);
     }
     // The copies into LDS are asm: the compiler would otherwise make every wave drain all of
     // its outstanding loads before the first LDS read behind the barrier, the weights it
     // prefetched two steps ahead included.  The wait before the barrier counts them instead.
     auto fetch_a = [&](uint32_t step, int buffer) {
+        const _Float16 *base = p.x + (size_t)step * kStepColumns;  // uniform
 #pragma unroll
         for (int j = 0; j < AJ; ++j) {
-            const uint32_t k = step * kStepColumns;
-            const uint32_t octet = r ^ (((BM / 4) * wave + 4u * j + kq) & 15u);
-            const _Float16 *source = a_source[j] + k;
-            if (k + 8u * octet >= p.K) source -= 64;
             const uint32_t lds_base =
                 (uint32_t)(uintptr_t)(lds_ptr)&a_lds[buffer][(BM / 4) * wave + 4u * j][0];
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :
-                         : "v"(source), "s"(lds_base)
+                         : "v"(a_offset[j]), "s"(base), "s"(lds_base)
                          : "memory");
         }
     };
     auto fetch_tile = [&](uint32_t step, uint32_t tile, uint4 &codes, uint2 &meta) {
         tile = tile < p.NT ? tile : p.NT - 1u;  // stay in bounds; such columns are never stored
-        const size_t record = (size_t)step * p.NT + tile;
-        codes = p.codes[record * 64u + lane];
-        meta = p.meta[record * 16u + r];
+        const size_t record = (size_t)step * p.NT + tile;  // uniform: scalar base, lane offset
+        codes = (p.codes + record * 64u)[lane];
+        meta = (p.meta + record * 16u)[r];
     };
     auto fetch_b = [&](uint32_t step, uint4 (&codes)[NTX], uint2 (&meta)[NTX]) {
 #pragma unroll
@@ -503,10 +502,12 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         __builtin_amdgcn_s_waitcnt(0x0070 | (2 * NTX));
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        fetch_a(clamp_step(step + 2u), buffer);
         quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), buffer ^ 1, b_codes[next],
                 b_meta[next]);
         __builtin_amdgcn_sched_barrier(0);
+        // after the quarter, so that the loads the compiler counts when it waits for the next
+        // step's weights are only the weight loads themselves
+        fetch_a(clamp_step(step + 2u), buffer);
         fetch_b(clamp_step(step + 3u), b_codes[cur], b_meta[cur]);
     };
     // whole rotations in a loop without branches (the compiler then counts the loads in flight
@@ -628,7 +629,10 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     int best = 0;
     uint32_t best_splits = 1;
     double best_cost = 1e30;
+    // the pipelined kernel addresses x with 32-bit byte offsets and whole 128-column steps
+    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * w.K * sizeof(_Float16) < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
+        if (v >= 6 && !pipe_ok) continue;
         const Variant &c = variants[v];
         const uint32_t tpb = 4u * c.ntw + c.extra;
         const uint32_t slots = cus * (uint32_t)c.resident;
@@ -666,7 +670,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     const char *force = getenv("MI355Q_Q4_GEMM");  // "VARIANT,SPLITS" for experiments
     int fv = 0, fs = 0;
     if (force && sscanf(force, "%d,%d", &fv, &fs) == 2 && fv >= 0 &&
-        fv < (int)(sizeof variants / sizeof variants[0]) && fs >= 1 && fs <= 16) {
+        fv < (int)(sizeof variants / sizeof variants[0]) && fs >= 1 && fs <= 16 && (fv < 6 || pipe_ok)) {
         best = fv;
         best_splits = (uint32_t)fs;
     }
