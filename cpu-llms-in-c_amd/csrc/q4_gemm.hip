@@ -292,8 +292,8 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
 // are asm statements: asm keeps its source order, which is what places each in its slot between
 // the matrix instructions; the caller keeps dependent stages at least one instruction apart,
 // which covers the wait state a packed-fp16 result needs before a vector instruction reads it.
-template <int STAGE, int PIECE, int D, int NTX>
-__device__ __forceinline__ void dequant_stage(const uint4 (&codes)[NTX], const uint2 (&meta)[NTX],
+template <int STAGE, int PIECE, int D, int NTX, class Codes, class Meta>
+__device__ __forceinline__ void dequant_stage(const Codes (&codes)[NTX], const Meta (&meta)[NTX],
                                               const NibbleMasks &masks, uint32_t (&merged)[4 * NTX],
                                               half2v (&centred)[4 * NTX], half2v (&out)[NTX][4])
 {
@@ -318,6 +318,56 @@ __device__ __forceinline__ void dequant_stage(const uint4 (&codes)[NTX], const u
     }
 }
 
+// Where the pipelined kernel puts the dequantization of one quarter among the SLOTS matrix
+// instructions of the previous one.  Slot k's vector instructions follow its matrix instruction
+// and, in the slots that end a fragment's use, the LDS read that refills it; phase(k) counts the
+// reads before them.  Piece p runs its stage s in phase first_phase(p) + s, and the
+// instructions of one phase are spread evenly over its slots.
+template <int MI, int NTW, int SLOTS, int PIECES, int LOADS>
+struct PipeSchedule {
+    // The LOADS global loads of one step's fetch are spread over four quarters (windows), evenly
+    // over the slots of each: a burst of them would fill the load queue and hold the wave.
+    static constexpr int window_of(int load) { return load * 4 / LOADS; }
+    static constexpr int load_at(int window, int k)
+    {
+        int members = 0;
+        for (int load = 0; load < LOADS; ++load) members += window_of(load) == window;
+        int index = 0;
+        for (int load = 0; load < LOADS; ++load)
+            if (window_of(load) == window) {
+                if ((2 * index + 1) * SLOTS / (2 * members) == k) return load;
+                ++index;
+            }
+        return -1;
+    }
+    static constexpr int window_loads(int window)
+    {
+        int members = 0;
+        for (int load = 0; load < LOADS; ++load) members += window_of(load) == window;
+        return members;
+    }
+    static constexpr int phase(int k) { return k < MI * NTW ? (k + 1) / NTW : MI + 1 + (k - MI * NTW); }
+    static constexpr int first_phase(int piece) { return piece * (MI - 1) / PIECES; }  // 0 .. MI-2
+    static constexpr int slot_of(int piece, int stage)
+    {
+        const int target = first_phase(piece) + stage;
+        int members = 0, index = 0;  // instructions of this phase, and this one's place among them
+        for (int other = 0; other < PIECES; ++other)
+            for (int s = 0; s < 3; ++s)
+                if (first_phase(other) + s == target) {
+                    if (other == piece && s == stage) index = members;
+                    ++members;
+                }
+        int first = -1, count = 0;  // slots of this phase
+        for (int k = 0; k < SLOTS; ++k)
+            if (phase(k) == target) {
+                if (first < 0) first = k;
+                ++count;
+            }
+        return first + index * count / members;
+    }
+};
+
 // One workgroup per compute unit, one wave per SIMD, software pipelined: while the
 // matrix instructions of one 32-column quarter run, the same wave dequantizes the
 // next quarter's weights and reads the next quarter's activation fragments from
@@ -326,15 +376,44 @@ __device__ __forceinline__ void dequant_stage(const uint4 (&codes)[NTX], const u
 // With XT the workgroup takes one tile more than its waves can split evenly
 // (4*NTW + 1, e.g. 17 = 1088 / 64): every wave dequantizes that tile and multiplies
 // it with its own quarter of the row fragments, so the four waves stay balanced.
+// Memory runs three steps ahead of the arithmetic: the activations of four steps
+// rotate through LDS (4 x 32 KiB, dynamic) and the weights of three through registers.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+constexpr uint32_t kPipeBuffers = 4;
+constexpr size_t pipe_lds_bytes(int bm) { return kPipeBuffers * (size_t)bm * 16u * sizeof(uint4); }
+
+// The pipelined kernel's global loads (uniform base + 32-bit lane offset), as asm: see there.
+template <int IMMEDIATE>
+__device__ __forceinline__ void load_to_lds(uint32_t lane_offset, const char *base, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2"
+                 :
+                 : "v"(lane_offset), "s"(base), "n"(IMMEDIATE), "s"(lds_base)
+                 : "memory");
+}
+__device__ __forceinline__ void load_x4(u32x4 &to, uint32_t lane_offset, const char *base)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(to) : "v"(lane_offset), "s"(base) : "memory");
+}
+__device__ __forceinline__ void load_x2(u32x2 &to, uint32_t lane_offset, const char *base)
+{
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(to) : "v"(lane_offset), "s"(base) : "memory");
+}
+
 template <int BM, int NTW, bool XT>
 __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p)
 {
-    __shared__ uint4 a_lds[2][BM][16];  // [buffer][row][slot], slot = octet ^ (row % 16)
+    extern __shared__ uint4 a_lds_raw[];  // [buffer][row][slot], slot = octet ^ (row % 16)
+    typedef uint4 (*stage_rows)[16];
+    auto a_lds = [&](uint32_t buffer) { return (stage_rows)(a_lds_raw + (size_t)buffer * BM * 16u); };
     constexpr int MI = BM / 16;  // 16-row fragments of x per workgroup
     constexpr int AJ = BM / 16;  // LDS-direct loads per wave per step (4 rows each)
     constexpr int TPB = 4 * NTW + (XT ? 1 : 0);
     constexpr int NTX = NTW + (XT ? 1 : 0);
     constexpr int XI = MI / 4;  // row fragments of the shared tile per wave
+    constexpr int GROUP = AJ + 2 * NTX;  // loads one step's fetch puts in flight
+    static_assert(2 * GROUP < 64, "the load counter holds 63");
     typedef __attribute__((address_space(3))) void *lds_ptr;
 
     const uint32_t lane = threadIdx.x & 63u;
@@ -349,43 +428,70 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
     if (step_begin >= step_end) return;  // uniform over the workgroup
 
-    // Activation stage.  The host sends only whole 128-column steps (K % 128 == 0) and
-    // M * K * 2 < 4 GiB here, so a lane's piece of the stage is one scalar base (advancing 256
-    // bytes per step) plus a 32-bit byte offset fixed for the whole kernel.  Rows beyond M
-    // re-read the last row: they stay in bounds and never reach y.
+    // Fetch addressing, arranged so that a step costs a handful of scalar instructions: one
+    // uniform pointer each into x, the codes and the metadata, advanced by one step per fetch,
+    // and per-lane 32-bit byte offsets fixed for the whole kernel (the host sends only whole
+    // 128-column steps, K % 128 == 0, and M * K * 2 < 4 GiB here).  Rows beyond M re-read the
+    // last row and tiles beyond NT the last tile: they stay in bounds and never reach y.
+    // The LDS-direct loads of a step share one M0: load j adds the immediate (j - AJ/2) * 1024
+    // to both the LDS and the global address, and its lane offset takes that back out of the
+    // latter (plus 4096, which the x pointer starts below x, so lane offsets stay positive).
+    static_assert(AJ == 8, "immediates -4096 .. 3072 cover eight loads");
     uint32_t a_offset[AJ];
 #pragma unroll
     for (int j = 0; j < AJ; ++j) {
         const uint32_t local = (BM / 4) * wave + 4u * j + kq;
         uint32_t m = m0 + local;
         m = m < p.M ? m : p.M - 1u;
-        a_offset[j] = (m * p.K + 8u * (r ^ (local & 15u))) * (uint32_t)sizeof(_Float16);
+        a_offset[j] = (m * p.K + 8u * (r ^ (local & 15u))) * (uint32_t)sizeof(_Float16) + 4096u -
+                      (uint32_t)((j - AJ / 2) * 1024);
     }
-    // The copies into LDS are asm: the compiler would otherwise make every wave drain all of
-    // its outstanding loads before the first LDS read behind the barrier, the weights it
-    // prefetched two steps ahead included.  The wait before the barrier counts them instead.
-    auto fetch_a = [&](uint32_t step, int buffer) {
-        const _Float16 *base = p.x + (size_t)step * kStepColumns;  // uniform
+    uint32_t codes_offset[NTX], meta_offset[NTX];
 #pragma unroll
-        for (int j = 0; j < AJ; ++j) {
-            const uint32_t lds_base =
-                (uint32_t)(uintptr_t)(lds_ptr)&a_lds[buffer][(BM / 4) * wave + 4u * j][0];
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :
-                         : "v"(a_offset[j]), "s"(base), "s"(lds_base)
-                         : "memory");
+    for (int t = 0; t < NTX; ++t) {
+        uint32_t tile = XT && t == NTX - 1 ? shared_tile : tile0 + t;
+        tile = tile < p.NT ? tile : p.NT - 1u;
+        codes_offset[t] = (tile * 64u + lane) * (uint32_t)sizeof(uint4);
+        meta_offset[t] = (tile * 16u + r) * (uint32_t)sizeof(uint2);
+    }
+    const uint32_t last_step = step_end - 1u;
+    // the fetch pointers: they stop at the last step (later fetches repeat it: no branches)
+    const char *x_next = (const char *)(p.x + (size_t)step_begin * kStepColumns) - 4096;
+    const char *codes_next = (const char *)(p.codes + (size_t)step_begin * p.NT * 64u);
+    const char *meta_next = (const char *)(p.meta + (size_t)step_begin * p.NT * 16u);
+    uint32_t fetch_step = step_begin;
+    const uint32_t codes_stride = p.NT * 64u * (uint32_t)sizeof(uint4);
+    const uint32_t meta_stride = p.NT * 16u * (uint32_t)sizeof(uint2);
+    const uint32_t lds_wave = (uint32_t)(uintptr_t)(lds_ptr)&a_lds(0)[(BM / 4) * wave][0] + 4096u;
+    // Every global load of the loop is an asm statement, so the compiler inserts no waits of
+    // its own for them (it would drain the whole queue before the first LDS read behind the
+    // barrier, prefetched steps included): the one wait before each step's barrier counts the
+    // loads that may stay in flight, and the registers a weight fetch fills are not read
+    // before the wait that covers it (`landed` below marks that point for the compiler).
+    // load number `load` of a step's fetch: the AJ pieces of the activation stage, then codes and
+    // metadata of each tile
+    auto fetch_one = [&](auto load_c, uint32_t buffer, u32x4 (&codes)[NTX], u32x2 (&meta)[NTX]) {
+        constexpr int load = decltype(load_c)::value;
+        if constexpr (load < AJ) {
+            const uint32_t lds_base = lds_wave + buffer * (uint32_t)(BM * 16u * sizeof(uint4));
+            load_to_lds<(load - AJ / 2) * 1024>(a_offset[load], x_next, lds_base);
+        } else if constexpr ((load - AJ) % 2 == 0) {
+            load_x4(codes[(load - AJ) / 2], codes_offset[(load - AJ) / 2], codes_next);
+        } else {
+            load_x2(meta[(load - AJ) / 2], meta_offset[(load - AJ) / 2], meta_next);
         }
     };
-    auto fetch_tile = [&](uint32_t step, uint32_t tile, uint4 &codes, uint2 &meta) {
-        tile = tile < p.NT ? tile : p.NT - 1u;  // stay in bounds; such columns are never stored
-        const size_t record = (size_t)step * p.NT + tile;  // uniform: scalar base, lane offset
-        codes = (p.codes + record * 64u)[lane];
-        meta = (p.meta + record * 16u)[r];
+    auto advance = [&]() {  // the pointers move on to the next step's fetch
+        const bool more = fetch_step < last_step;
+        fetch_step += 1u;
+        x_next += more ? kStepColumns * sizeof(_Float16) : 0u;
+        codes_next += more ? codes_stride : 0u;
+        meta_next += more ? meta_stride : 0u;
     };
-    auto fetch_b = [&](uint32_t step, uint4 (&codes)[NTX], uint2 (&meta)[NTX]) {
+    // after the wait that covers their fetch: from here on the registers hold the weights
+    auto landed = [&](u32x4 (&codes)[NTX], u32x2 (&meta)[NTX]) {
 #pragma unroll
-        for (int t = 0; t < NTW; ++t) fetch_tile(step, tile0 + t, codes[t], meta[t]);
-        if (XT) fetch_tile(step, shared_tile, codes[NTX - 1], meta[NTX - 1]);
+        for (int t = 0; t < NTX; ++t) asm volatile("" : "+v"(codes[t]), "+v"(meta[t]));
     };
     const NibbleMasks masks = nibble_masks();
 
@@ -398,27 +504,26 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
 #pragma unroll
     for (int i = 0; i < XI; ++i) acc_shared[i] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // Steady state of one step (buffer = step parity):
-    //   quarters 0..2: matrix instructions of quarter d | LDS reads + dequantization of d+1
-    //   wait for the fetches of step+1, barrier (all waves hold their last fragments of
-    //   this buffer in registers, so it may be refilled)
-    //   quarter 3: fetch step+2 | matrix instructions | reads + dequantization of quarter 0
-    //   of step+1 from the other buffer.
-    // Steps past the end are clamped to the last one (a redundant fetch, no branches).
+    // Steady state of one step (buffer = step % 4, weight registers = step % 3):
+    //   quarters 0..2: matrix instructions of quarter d | LDS reads + dequantization of d+1 |
+    //   second to fourth quarter of the fetch of step+2
+    //   wait until only that fetch is in flight, barrier: the activations and weights of
+    //   step+1 have landed for every wave
+    //   quarter 3: matrix instructions | reads + dequantization of quarter 0 of step+1 | first
+    //   quarter of the fetch of step+3: activations into the buffer of step-1 (every wave
+    //   consumed its last fragments of it before the barrier it just passed), weights into
+    //   this step's registers.
+    // Fetches past the end repeat the last step (redundant, no branches).
     // The matrix instructions are written as asm with the accumulator tied in place (in the
     // accumulation registers); a scheduling barrier after each pins the few vector
     // instructions and the LDS read that follow it in the source to that slot.
-    const uint32_t last_step = step_end - 1u;
-    auto clamp_step = [&](uint32_t step) { return step < last_step ? step : last_step; };
-    // three register sets of codes and metadata, in rotation: the step being multiplied, the
-    // next one, and the one after that still in flight (weights come from HBM: two steps of lead)
-    uint4 b_codes[3][NTX];
-    uint2 b_meta[3][NTX];
+    u32x4 b_codes[3][NTX];
+    u32x2 b_meta[3][NTX];
     half2v b_frag[2][NTX][4];  // [set][tile][column pair group]: 8 weights of a lane
     half8 a_frag[MI];
     half8 a_shared[XI];
-    auto read_frag = [&](int buffer, int d, uint32_t fragment) {
-        return __builtin_bit_cast(half8, a_lds[buffer][16 * fragment + r][(4 * d + kq) ^ r]);
+    auto read_frag = [&](uint32_t buffer, int d, uint32_t fragment) {
+        return __builtin_bit_cast(half8, a_lds(buffer)[16 * fragment + r][(4 * d + kq) ^ r]);
     };
     auto multiply = [&](floatx4 &c, const half8 &a, const half2v (&b)[4]) {
         const half8 b8 = {b[0].x, b[0].y, b[1].x, b[1].y, b[2].x, b[2].y, b[3].x, b[3].y};
@@ -427,20 +532,23 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     // Dequantization of one quarter = NTX tiles x 4 pieces (two of a lane's eight weights each),
     // each piece three dependent vector instructions: mask-and-merge into an fp16 with the code in
     // its mantissa, subtract the offset, fused multiply-add with the group's {scale, bias}.
-    // Piece p starts in slot p * (SLOTS - 3) / PIECES and advances one stage per slot, so no slot holds two
-    // dependent instructions back to back.
+    // They are asm statements (asm keeps its source order, which is what places each in its slot
+    // behind a matrix instruction).  The compiler pads two dependent asm statements with a no-op
+    // unless an instruction of its own stands between them, so the three stages of a piece sit
+    // in three consecutive phases of the quarter, a phase being the slots between two of the LDS
+    // reads that refill the fragments (one every NTW slots): no padding, and the distance also
+    // covers the wait state a packed-fp16 result needs before a vector instruction reads it.
     constexpr int SLOTS = MI * NTW + (XT ? XI : 0);
     constexpr int PIECES = 4 * NTX;
-    // The three instructions are asm statements: asm keeps its source order, which is what
-    // places each of them in its slot, and the slot distance between dependent ones also covers
-    // the one wait state a packed-fp16 result needs before the next vector instruction reads it.
+    typedef PipeSchedule<MI, NTW, SLOTS, PIECES, GROUP> Schedule;
     uint32_t merged[PIECES];
     half2v centred[PIECES];
     // One quarter: the matrix instructions on b_frag[cur] and the resident fragments; between
     // them the dequantization of quarter next_d (of `codes`) into b_frag[cur ^ 1] and the
     // refill of every fragment, right after its last use, with quarter next_d of next_buffer.
-    auto quarter = [&](auto cur_c, auto next_d_c, int next_buffer, const uint4 (&codes)[NTX],
-                       const uint2 (&meta)[NTX]) {
+    auto quarter = [&](auto cur_c, auto next_d_c, uint32_t next_buffer, const u32x4 (&codes)[NTX],
+                       const u32x2 (&meta)[NTX], auto window_c, uint32_t fetch_buffer,
+                       u32x4 (&fetch_codes)[NTX], u32x2 (&fetch_meta)[NTX]) {
         constexpr int cur = decltype(cur_c)::value;
         static_for<SLOTS>([&](auto k_c) {
             constexpr int k = decltype(k_c)::value;
@@ -455,22 +563,37 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
             }
             static_for<PIECES>([&](auto piece_c) {
                 constexpr int piece = decltype(piece_c)::value;
-                constexpr int stage = k - piece * (SLOTS - 3) / PIECES;
-                if constexpr (stage >= 0 && stage < 3)
-                    dequant_stage<stage, piece, decltype(next_d_c)::value>(codes, meta, masks, merged,
-                                                                           centred, b_frag[cur ^ 1]);
+                static_for<3>([&](auto stage_c) {
+                    constexpr int stage = decltype(stage_c)::value;
+                    if constexpr (Schedule::slot_of(piece, stage) == k)
+                        dequant_stage<stage, piece, decltype(next_d_c)::value>(codes, meta, masks, merged,
+                                                                               centred, b_frag[cur ^ 1]);
+                });
             });
+            constexpr int load = Schedule::load_at(decltype(window_c)::value, k);
+            if constexpr (load >= 0)
+                fetch_one(std::integral_constant<int, load>(), fetch_buffer, fetch_codes, fetch_meta);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    // s_waitcnt immediate: at most `loads` global loads in flight, LDS and scalar traffic not
+    // waited for (load count: bits 3:0 and 15:14)
+    auto wait_loads = [](auto loads_c) {
+        constexpr int loads = decltype(loads_c)::value;
+        __builtin_amdgcn_s_waitcnt((loads & 15) | ((loads >> 4) << 14) | 0x0f70);
+    };
 
-    fetch_a(step_begin, 0);
-    fetch_b(step_begin, b_codes[0], b_meta[0]);
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    fetch_a(clamp_step(step_begin + 1u), 1);
-    fetch_b(clamp_step(step_begin + 1u), b_codes[1], b_meta[1]);
-    fetch_b(clamp_step(step_begin + 2u), b_codes[2], b_meta[2]);
+    static_for<GROUP>([&](auto load_c) { fetch_one(load_c, 0, b_codes[0], b_meta[0]); });
+    advance();
+    static_for<GROUP>([&](auto load_c) { fetch_one(load_c, 1, b_codes[1], b_meta[1]); });
+    advance();
+    static_for<GROUP>([&](auto load_c) {
+        if constexpr (Schedule::window_of(decltype(load_c)::value) == 0) fetch_one(load_c, 2, b_codes[2], b_meta[2]);
+    });
+    wait_loads(std::integral_constant<int, GROUP + Schedule::window_loads(0)>());
+    landed(b_codes[0], b_meta[0]);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < MI; ++i) a_frag[i] = read_frag(0, 0, i);
     if (XT) {
@@ -485,33 +608,36 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         });
     });
 
-    // One step with the register set `cur` (this step's weights) and `next` (the next step's);
-    // `cur` is free after quarter 2 and receives the weights of step + 3.
+    // One step with the register sets `cur` (this step's weights), `next` (the next step's) and
+    // the third, which quarters 0..2 fill with the weights of step + 2 (the rest of the fetch
+    // that quarter 3 of the previous step began); `cur` is free after quarter 2, and quarter 3
+    // begins the fetch of step + 3 into it.
     auto one_step = [&](uint32_t step, auto cur_c, auto next_c) {
         constexpr int cur = decltype(cur_c)::value, next = decltype(next_c)::value;
-        const int buffer = (int)((step - step_begin) & 1u);
+        constexpr int third = 3 - cur - next;
+        const uint32_t buffer = (step - step_begin) % kPipeBuffers;
         static_for<3>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
             __builtin_amdgcn_sched_barrier(0);
             quarter(std::integral_constant<int, (d & 1)>(), std::integral_constant<int, d + 1>(), buffer,
-                    b_codes[cur], b_meta[cur]);
+                    b_codes[cur], b_meta[cur], std::integral_constant<int, d + 1>(),
+                    (buffer + 2u) % kPipeBuffers, b_codes[third], b_meta[third]);
         });
         __builtin_amdgcn_sched_barrier(0);
-        // everything but the newest weight fetch (2 * NTX loads, of step + 2) has landed: the
-        // activations and weights of step + 1; and this wave's LDS reads are done
-        __builtin_amdgcn_s_waitcnt(0x0070 | (2 * NTX));
-        __syncthreads();
+        advance();
+        // only the fetch of step + 2, just completed, may still be in flight
+        wait_loads(std::integral_constant<int, GROUP>());
+        landed(b_codes[next], b_meta[next]);
+        // no wait for this wave's LDS reads: the buffer refilled next is one whose last
+        // fragments every wave had consumed before it reached this barrier
+        __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), buffer ^ 1, b_codes[next],
-                b_meta[next]);
+        quarter(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), (buffer + 1u) % kPipeBuffers,
+                b_codes[next], b_meta[next], std::integral_constant<int, 0>(), (buffer + 3u) % kPipeBuffers,
+                b_codes[cur], b_meta[cur]);
         __builtin_amdgcn_sched_barrier(0);
-        // after the quarter, so that the loads the compiler counts when it waits for the next
-        // step's weights are only the weight loads themselves
-        fetch_a(clamp_step(step + 2u), buffer);
-        fetch_b(clamp_step(step + 3u), b_codes[cur], b_meta[cur]);
     };
-    // whole rotations in a loop without branches (the compiler then counts the loads in flight
-    // exactly), the last one or two steps after it
+    // whole rotations of the three register sets in a loop, the last one or two steps after it
     uint32_t step = step_begin;
     for (; step + 3u <= step_end; step += 3u) {
         one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
@@ -522,7 +648,13 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     if (step + 1u < step_end)
         one_step(step + 1u, std::integral_constant<int, 1>(), std::integral_constant<int, 2>());
 
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // the last step's spare fetch into LDS has landed
+    // The spare fetches of the last steps land in LDS and in registers nobody reads: those
+    // registers stay reserved until the loads are back.
+    __builtin_amdgcn_sched_barrier(0);
+    wait_loads(std::integral_constant<int, 0>());
+#pragma unroll
+    for (int set = 0; set < 3; ++set) landed(b_codes[set], b_meta[set]);
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- lane (r, kq) holds rows 16*i + 4*kq + j of column tile*16 + r
     auto store_all = [&](auto mode) {
@@ -575,6 +707,24 @@ q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__re
     const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (index >= count) return;
     out[index] = (_Float16)load_as_float(x, x_dtype, index);
+}
+
+// The pipelined kernel's stage is larger than the 64 KiB a kernel gets without asking: the
+// limit is raised once per device and instantiation.
+template <bool XT>
+static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &p)
+{
+    static bool raised[64] = {};
+    constexpr size_t bytes = pipe_lds_bytes(128);
+    const int device = ctx->device;
+    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+    if (!raised[device]) {
+        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, 4, XT>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (status != hipSuccess) return status;
+        raised[device] = true;
+    }
+    return launch(ctx, q4_gemm_pipe_kernel<128, 4, XT>, grid, dim3(256), bytes, p);
 }
 
 int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
@@ -701,8 +851,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     case 3: launched = launch(ctx, q4_gemm_kernel<64, 4, true>, grid, dim3(256), 0, p); break;
     case 4: launched = launch(ctx, q4_gemm_kernel<64, 2, false>, grid, dim3(256), 0, p); break;
     case 5: launched = launch(ctx, q4_gemm_kernel<64, 2, true>, grid, dim3(256), 0, p); break;
-    case 6: launched = launch(ctx, q4_gemm_pipe_kernel<128, 4, false>, grid, dim3(256), 0, p); break;
-    default: launched = launch(ctx, q4_gemm_pipe_kernel<128, 4, true>, grid, dim3(256), 0, p); break;
+    case 6: launched = launch_pipe<false>(ctx, grid, p); break;
+    default: launched = launch_pipe<true>(ctx, grid, p); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);
