@@ -383,6 +383,19 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr uint32_t kPipeBuffers = 4;
 constexpr size_t pipe_lds_bytes(int bm) { return kPipeBuffers * (size_t)bm * 16u * sizeof(uint4); }
 
+// An empty statement that uses and redefines a register: the compiler must have the value
+// ready here (it waits for the load that produces it) and reads it no earlier afterwards.
+template <class T>
+__device__ __forceinline__ void touch(T &a, T &b)
+{
+    asm volatile("" : "+v"(a), "+v"(b));
+}
+template <class T>
+__device__ __forceinline__ void touch(T &a, T &b, T &c, T &d)
+{
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+
 // The pipelined kernel's global loads (uniform base + 32-bit lane offset), as asm: see there.
 template <int IMMEDIATE>
 __device__ __forceinline__ void load_to_lds(uint32_t lane_offset, const char *base, uint32_t lds_base)
@@ -525,6 +538,13 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     auto read_frag = [&](uint32_t buffer, int d, uint32_t fragment) {
         return __builtin_bit_cast(half8, a_lds(buffer)[16 * fragment + r][(4 * d + kq) ^ r]);
     };
+    static_assert(MI == 8 && XI == 2, "the groups of fragments waited for together");
+    auto touch_frags = [&](auto from_c, auto to_c) {
+        constexpr int from = decltype(from_c)::value;
+        static_assert(decltype(to_c)::value - from == 4, "four fragments per group");
+        touch(a_frag[from], a_frag[from + 1], a_frag[from + 2], a_frag[from + 3]);
+    };
+    auto touch_shared = [&]() { touch(a_shared[0], a_shared[1]); };
     auto multiply = [&](floatx4 &c, const half8 &a, const half2v (&b)[4]) {
         const half8 b8 = {b[0].x, b[0].y, b[1].x, b[1].y, b[2].x, b[2].y, b[3].x, b[3].y};
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b8));
@@ -555,10 +575,18 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
             if constexpr (k < MI * NTW) {
                 constexpr int i = k / NTW, t = k % NTW;
                 multiply(acc[i][t], a_frag[i], b_frag[cur][t]);
+                // One wait per group of fragments instead of one per fragment: the compiler waits
+                // where a loaded register is first used, and these empty statements use a whole
+                // group at once, one slot (and one LDS read) before its first matrix
+                // instruction; the reads waited for are at least half a quarter old.
+                if constexpr (k == MI / 2 * NTW - 1) touch_frags(std::integral_constant<int, MI / 2>(), std::integral_constant<int, MI>());
+                if constexpr (XT && k == MI * NTW - 1) touch_shared();
+                if constexpr (k == SLOTS - 1) touch_frags(std::integral_constant<int, 0>(), std::integral_constant<int, MI / 2>());
                 if constexpr (t == NTW - 1) a_frag[i] = read_frag(next_buffer, decltype(next_d_c)::value, i);
             } else {
                 constexpr int i = k - MI * NTW;
                 multiply(acc_shared[i], a_shared[i], b_frag[cur][NTX - 1]);
+                if constexpr (k == SLOTS - 1) touch_frags(std::integral_constant<int, 0>(), std::integral_constant<int, MI / 2>());
                 a_shared[i] = read_frag(next_buffer, decltype(next_d_c)::value, XI * wave + i);
             }
             static_for<PIECES>([&](auto piece_c) {
