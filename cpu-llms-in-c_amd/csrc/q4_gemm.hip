@@ -788,21 +788,22 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
 
     // Decomposition: BM rows x (4*NTW + EXTRA) tiles per workgroup, K split in `splits`.
     // The choice minimises a microsecond estimate fitted to sweeps over every variant
-    // and split on this GPU: a workgroup that has a compute unit to itself sustains
-    // `alone` of the matrix-instruction peak, co-resident workgroups `shared` together;
-    // a grid that is not a whole number of resident sets pays ~0.3 of a workgroup time for
-    // its ragged end, and a K split pays for its fp32 partials at ~4.3 TB/s.
+    // and split on this GPU.  Kernels 0-5: a workgroup that has a compute unit to itself
+    // sustains `alone` of the matrix-instruction peak, co-resident workgroups `shared`
+    // together; a grid that is not a whole number of resident sets pays ~0.3 of a workgroup
+    // time for its ragged end.  The pipelined kernel (6, 7; one workgroup per compute unit)
+    // runs in whole rounds of `alone` of the peak plus `round_us` each.  A K split pays for
+    // its fp32 partials at ~4 TB/s.
     struct Variant {
         int bm, ntw, extra;
         int resident;          // workgroups that fit one compute unit (registers, LDS)
         double alone, shared;  // fraction of matrix-instruction peak, one / several per CU
+        double round_us;       // pipelined kernel: fixed time per round of workgroups
     };
-    // 0-5: two workgroups per compute unit overlap each other; 6, 7: the pipelined kernel,
-    // one workgroup per compute unit
-    static const Variant variants[] = {{128, 4, 0, 2, 0.412, 0.502}, {128, 2, 0, 2, 0.350, 0.463},
-                                       {64, 4, 0, 3, 0.358, 0.478},  {64, 4, 1, 2, 0.385, 0.470},
-                                       {64, 2, 0, 4, 0.350, 0.443},  {64, 2, 1, 2, 0.399, 0.473},
-                                       {128, 4, 0, 1, 0.476, 0.450}, {128, 4, 1, 1, 0.445, 0.430}};
+    static const Variant variants[] = {
+        {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
+        {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
+        {128, 4, 0, 1, 0.685, 0.685, 13.0}, {128, 4, 1, 1, 0.654, 0.654, 16.5}};
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     int best = 0;
     uint32_t best_splits = 1;
@@ -826,7 +827,14 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             const double tiles_per_wave = v >= 6 ? c.ntw + 0.25 * c.extra : c.ntw + c.extra;
             const double peak_us = (double)steps * tiles_per_wave * (c.bm / 16.0) * 64.0 / 2400.0;
             double cost;
-            if (groups <= cus)
+            if (v >= 6) {
+                // a last round that leaves compute units idle runs at a higher clock (power)
+                const double round = peak_us / c.alone;
+                const uint64_t rest = groups % cus;
+                cost = (double)(groups / cus) * (round + c.round_us) +
+                       (rest ? round * (0.8 + 0.2 * rest / cus) + c.round_us : 0.0);
+            }
+            else if (groups <= cus)
                 cost = peak_us / c.alone;
             else if (groups <= slots) {
                 // k of the `resident` workgroups a compute unit could hold: in between
@@ -835,9 +843,9 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
                 cost = k * peak_us / sustained;
             }
             else
-                cost = ((double)groups / slots + (groups % slots ? 0.29 : 0.0)) * c.resident * peak_us / c.shared;
+                cost = ((double)groups / slots + (groups % slots ? 0.31 : 0.0)) * c.resident * peak_us / c.shared;
             if (splits > 1)  // fp32 partials written and read back
-                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.3e12 * 1.0e6;
+                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.0e12 * 1.0e6;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;
