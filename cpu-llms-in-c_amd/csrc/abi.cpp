@@ -498,6 +498,84 @@ int mi355q_q4_dequant_rows(mi355q_context *ctx, const mi355q_q4_weight *weight, 
     return MI355Q_OK;
 }
 
+int mi355q_q4_linear_rows(mi355q_context *ctx, const mi355q_q4_weight *weight, const uint32_t *rows,
+                          uint32_t count, const void *x, int x_dtype, uint32_t M, void *y, int y_dtype,
+                          uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || x == nullptr || y == nullptr || count == 0 || M == 0 ||
+        !dtype_valid(x_dtype) || !dtype_valid(y_dtype)) {
+        set_error(error, error_capacity, "q4_linear_rows: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "q4_linear_rows: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    const Q4Device &dev = weight->dev;
+    if ((x_dtype == MI355Q_F32 ? 2u * M : M) > 16u) {
+        set_error(error, error_capacity, "q4_linear_rows: at most 16 activation rows (8 of fp32), got %u", M);
+        return MI355Q_ERROR_INVALID;
+    }
+    const bool x_dev = flags & MI355Q_X_DEVICE, y_dev = flags & MI355Q_Y_DEVICE;
+    const bool rows_dev = rows == nullptr || (flags & MI355Q_SOURCE_DEVICE);
+    if ((flags & MI355Q_ASYNC) && !(x_dev && y_dev && rows_dev)) {
+        set_error(error, error_capacity, "q4_linear_rows: ASYNC needs device pointers throughout");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (x_dev && ((uintptr_t)x & 15u) != 0) {
+        set_error(error, error_capacity, "q4_linear_rows: device x must be 16-byte aligned");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (rows == nullptr && count > dev.N) {
+        set_error(error, error_capacity, "q4_linear_rows: the first %u rows of a %u-row matrix", count, dev.N);
+        return MI355Q_ERROR_INVALID;
+    }
+    if (rows != nullptr && !rows_dev)
+        for (uint32_t i = 0; i < count; ++i)
+            if (rows[i] >= dev.N) {
+                set_error(error, error_capacity, "q4_linear_rows: row %u of a %u-row matrix", rows[i], dev.N);
+                return MI355Q_ERROR_INVALID;
+            }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t x_bytes = (size_t)M * dev.K * dtype_bytes(x_dtype);
+    const size_t y_bytes = (size_t)M * count * dtype_bytes(y_dtype);
+    const size_t row_bytes = (size_t)count * sizeof(uint32_t);
+    Q4LinearArgs args;
+    memset(&args, 0, sizeof args);
+    args.x = x;
+    args.x_dtype = x_dtype;
+    args.M = M;
+    args.y_dtype = y_dtype;
+    args.count = 1;
+    args.targets[0].w = &dev;
+    args.targets[0].y = y;
+    args.row_ids = rows;
+    args.row_count = count;
+    int status;
+    if (!x_dev) {
+        if ((status = ensure_stage(ctx, 0, x_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[0], x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "activation upload");
+        args.x = ctx->stage[0];
+    }
+    if (!y_dev) {
+        if ((status = ensure_stage(ctx, 1, y_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        args.targets[0].y = ctx->stage[1];
+    }
+    if (!rows_dev) {
+        if ((status = ensure_stage(ctx, 2, row_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[2], rows, row_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "row id upload");
+        args.row_ids = (const uint32_t *)ctx->stage[2];
+    }
+    if ((status = q4_stream_linear(ctx, args, error, error_capacity)) != MI355Q_OK) return status;
+    if (!y_dev)
+        MI355Q_HIP(hipMemcpyAsync(y, args.targets[0].y, y_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                   "output download");
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear_rows sync");
+    return MI355Q_OK;
+}
+
 int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count,
                            const void *x, int x_dtype, uint32_t M, int y_dtype, int residual_dtype,
                            uint32_t flags, char *error, size_t error_capacity)

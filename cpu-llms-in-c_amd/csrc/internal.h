@@ -144,6 +144,10 @@ struct Q4LinearArgs {
     int residual_dtype;
     bool residual_is_bias;  // residual is one row [N] added to every activation row
     bool fuse_silu;         // targets = {gate, up}: y[0] = silu(gate . x) * (up . x)
+    // a subset of the rows of the one target: output column j is row row_ids[j] (device
+    // pointer), or row j when row_ids is null; y is [M][row_count].  0 = all rows.
+    const uint32_t *row_ids;
+    uint32_t row_count;
     uint32_t count;
     Q4Target targets[kMaxTargets];
 };

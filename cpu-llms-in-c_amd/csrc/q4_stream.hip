@@ -40,6 +40,11 @@ struct StreamParams {
     void *y[kMaxTargets];
     const void *residual[kMaxTargets];
     uint32_t N[kMaxTargets], NT[kMaxTargets], first_block[kMaxTargets];
+    uint32_t stride[kMaxTargets];  // tiles per step in memory (NT unless a subset of the rows is computed)
+    // Row subset (one target): output column j is row ids[j] of the matrix, which has
+    // matrix_rows rows; N and NT then describe the outputs.  Null: column j is row j.
+    const uint32_t *ids;
+    uint32_t matrix_rows;
     uint32_t targets;
     const _Float16 *x;  // [rows][K] fp16
     uint32_t M, K, T;
@@ -87,7 +92,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 #pragma unroll
     for (uint32_t t = 1; t < kMaxTargets; ++t)
         if (t < p.targets && blockIdx.x >= p.first_block[t]) target = t;
-    const uint32_t NT = p.NT[target], N = p.N[target];
+    const uint32_t NT = p.NT[target], N = p.N[target], stride = p.stride[target];
     // tiles per target and workgroup: TB, or TB/2 of each of the two fused targets
     const uint32_t span_tiles = p.fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
     const uint32_t tile0 = (blockIdx.x - p.first_block[target]) * span_tiles;
@@ -104,6 +109,17 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         const uint32_t slot_target = p.fuse_silu ? (uint32_t)tb / span_tiles : target;
         uint32_t tile = tile0 + (uint32_t)tb % span_tiles;
         tile = tile < NT ? tile : NT - 1u;
+        if (p.ids != nullptr) {
+            // gathered rows: lane (r, kq) streams row ids[16*tile + r] out of whichever tile holds
+            // it (a slot or an id beyond the end re-reads a valid row; its result is not used)
+            uint32_t slot = tile * kTileRows + r;
+            slot = slot < N ? slot : N - 1u;
+            uint32_t row = p.ids[slot];
+            row = row < p.matrix_rows ? row : p.matrix_rows - 1u;
+            codes_tile[tb] = p.codes[slot_target] + (size_t)(row / kTileRows) * 64u + kq * 16u + row % kTileRows;
+            meta_tile[tb] = p.meta[slot_target] + (size_t)(row / kTileRows) * 16u + row % kTileRows;
+            continue;
+        }
         codes_tile[tb] = p.codes[slot_target] + (size_t)tile * 64u + lane;
         meta_tile[tb] = p.meta[slot_target] + (size_t)tile * 16u + r;
     }
@@ -131,8 +147,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             const uint32_t step = step0 + i * W;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * NT * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * NT * 16u);
+                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * stride * 64u);
+                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * stride * 16u);
             }
         };
         auto issue_clamped = [&](uint32_t i, StepData<TB> &slot) {
@@ -141,8 +157,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             step = step < p.T ? step : p.T - 1u;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * NT * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * NT * 16u);
+                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * stride * 64u);
+                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * stride * 16u);
             }
         };
         // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
@@ -293,6 +309,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             }
             if (p.residual[target])
                 value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
+            if (p.ids != nullptr && p.ids[n] >= p.matrix_rows) value = 0.0f;  // no such row
             store_from_float(p.y[target], p.y_dtype, at, value);
         }
     }
@@ -324,6 +341,7 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
     }
     if (p.residual[target])
         value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
+    if (p.ids != nullptr && p.ids[n] >= p.matrix_rows) value = 0.0f;  // no such row
     store_from_float(p.y[target], p.y_dtype, at, value);
 }
 
@@ -476,8 +494,16 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = (const _Float16 *)ctx->stage[3];
     }
+    const bool subset = a.row_count != 0u;
+    if (subset && (a.count != 1u || a.fuse_silu || a.targets[0].residual != nullptr ||
+                   (a.row_ids == nullptr && a.row_count > first.N))) {
+        set_error(error, error_capacity, "q4 stream kernel: a row subset takes one weight, no residual, and a "
+                                         "prefix no longer than the matrix");
+        return MI355Q_ERROR_INVALID;
+    }
     uint32_t tiles = 0;
-    for (uint32_t t = 0; t < a.count; ++t) tiles += a.targets[t].w->NT;
+    for (uint32_t t = 0; t < a.count; ++t)
+        tiles += subset ? (a.row_count + kTileRows - 1) / kTileRows : a.targets[t].w->NT;
     StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
     if (a.fuse_silu && shape.tb != 2 && shape.tb != 4) shape.tb = 2;  // gate and up tiles pair up
     uint32_t block = 0;
@@ -487,13 +513,16 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         p.meta[t] = w.meta;
         p.y[t] = a.targets[t].y;
         p.residual[t] = a.targets[t].residual;
-        p.N[t] = w.N;
-        p.NT[t] = w.NT;
+        p.N[t] = subset ? a.row_count : w.N;
+        p.NT[t] = subset ? (a.row_count + kTileRows - 1) / kTileRows : w.NT;
+        p.stride[t] = w.NT;
         p.first_block[t] = block;
-        block += (w.NT + shape.tb - 1) / shape.tb;
+        block += (p.NT[t] + shape.tb - 1) / shape.tb;
     }
     if (a.fuse_silu) p.first_block[1] = 0xffffffffu;  // every workgroup starts from target 0
     p.fuse_silu = a.fuse_silu;
+    p.ids = subset ? a.row_ids : nullptr;
+    p.matrix_rows = first.N;
     p.targets = a.count;
     p.M = a.M;
     p.K = first.K;
@@ -505,7 +534,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     if (p.slices > 1u) {
         for (uint32_t t = 0; t < a.count; ++t) {
             p.n_first[t] = p.n_total;
-            p.n_total += a.targets[t].w->N;
+            p.n_total += p.N[t];
         }
         int status = ensure_stage(ctx, 4, (size_t)p.slices * a.M * p.n_total * sizeof(float), error,
                                   error_capacity);

@@ -76,6 +76,7 @@ SIGNATURES = {
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
+    "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_multi": (_int, [_vp, _c.POINTER(Q4Target), _u32, _vp, _int, _u32, _int, _int,
                                       _u32, *_err]),
@@ -278,6 +279,26 @@ class Context:
               _ptr(y), y_dtype, _ptr(residual), residual_dtype,
               RESIDUAL_IS_BIAS if residual_is_bias else 0)
         return y
+
+    def q4_linear_rows(self, weight: Q4Weight, rows, x: np.ndarray, x_dtype: int, y_dtype: int = F32,
+                       count: int | None = None) -> np.ndarray:
+        """The linear restricted to output rows `rows` (ids), or to the first `count` rows when
+        rows is None: x [M][K] -> y [M][len(rows) or count]."""
+        x = np.ascontiguousarray(x)
+        M = x.shape[0]
+        if rows is not None:
+            rows = np.ascontiguousarray(rows, dtype=np.uint32)
+            count = rows.size
+        y = np.empty((M, count), dtype=_NP_DTYPE[y_dtype])
+        _call(self.lib.mi355q_q4_linear_rows, self.handle, weight.handle, _ptr(rows), count, _ptr(x), x_dtype,
+              M, _ptr(y), y_dtype, 0)
+        return y
+
+    def q4_linear_rows_device(self, weight: Q4Weight, rows_ptr: int | None, count: int, x_ptr: int,
+                              x_dtype: int, M: int, y_ptr: int, y_dtype: int, asynchronous: bool = True):
+        flags = X_DEVICE | Y_DEVICE | SOURCE_DEVICE | (ASYNC if asynchronous else 0)
+        _call(self.lib.mi355q_q4_linear_rows, self.handle, weight.handle, rows_ptr, count, x_ptr, x_dtype, M,
+              y_ptr, y_dtype, flags)
 
     def q4_gate_up_silu(self, gate: Q4Weight, up: Q4Weight, x: np.ndarray, x_dtype: int,
                         y_dtype: int = F32) -> np.ndarray:

@@ -207,6 +207,20 @@ int mi355q_q4_dequant_rows(mi355q_context *ctx, const mi355q_q4_weight *weight,
                            const uint32_t *rows, uint32_t count, void *out, int out_dtype,
                            uint32_t flags, char *error, size_t error_capacity);
 
+/* y[m][j] = (row rows[j] of the weight) . x[m], j < count, for 1..16 activation rows (8 of
+ * fp32): the linear restricted to some of its output rows.  rows == NULL takes the
+ * first `count` rows (count <= N).  This is the reference's restricted-vocabulary draft head:
+ * qwen38_q4_lm_head over a static low-id prefix of the vocabulary and
+ * qwen38_q4_lm_head_gathered over a list of further token ids (qwen38_global.metal:39-96).
+ * The weight bytes of the selected rows are read once; the arithmetic is that of
+ * mi355q_q4_linear.  MI355Q_X_DEVICE / MI355Q_Y_DEVICE as there; MI355Q_SOURCE_DEVICE: `rows`
+ * is a device pointer (an id past the matrix then yields 0; host ids are checked and
+ * rejected with status 2).  MI355Q_ASYNC needs all three on the device. */
+int mi355q_q4_linear_rows(mi355q_context *ctx, const mi355q_q4_weight *weight,
+                          const uint32_t *rows, uint32_t count, const void *x, int x_dtype,
+                          uint32_t M, void *y, int y_dtype, uint32_t flags,
+                          char *error, size_t error_capacity);
+
 /* y[m][n] = sum_k w[n][k] * x[m][k]  (+ residual[m][n] when residual != NULL)
  *
  * x: [M][K] of x_dtype (F16, F32 or BF16); y: [M][N] of y_dtype; residual:

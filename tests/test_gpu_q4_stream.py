@@ -249,6 +249,44 @@ def test_lm_head_sized_gemv(engine, oracle, gpu):
         assert q4_relative_error(y[:, begin:begin + 48], ref) <= TOLERANCE
 
 
+@pytest.mark.parametrize("M,x_dtype,meta_kind", [(1, "F16", "META_F16_INTERLEAVED"), (4, "F16", "META_BF16_PLANES"),
+                                                 (8, "F16", "META_BF16_PLANES"), (2, "F32", "META_BF16_PLANES")])
+def test_row_subsets(engine, oracle, gpu, M, x_dtype, meta_kind):
+    """mi355q_q4_linear_rows, the restricted-vocabulary head (qwen38_q4_lm_head over a low-id
+    prefix, qwen38_q4_lm_head_gathered over listed ids; qwen38_global.metal:39-96): a prefix
+    that ends inside a tile and a gathered list (unsorted, with repeats, first and last row,
+    a count that is no multiple of 16) must equal the same rows of the full linear, and the
+    oracle on those rows, to the usual tolerance.  K=8704 is cut in slices at M=8."""
+    x_dtype, meta_kind = getattr(engine, x_dtype), getattr(engine, meta_kind)
+    N, K = 1000, 8704 if M == 8 else 1536
+    quants, meta_a, meta_b = engine.synth_q4_affine(31, 0.02, N, K, meta_kind)
+    x = make_x(engine, 32, M, K, x_dtype)
+    rng = np.random.default_rng(33)
+    ids = np.concatenate([[N - 1, 0, 17, 17], rng.integers(0, N, size=71)]).astype(np.uint32)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, meta_kind)
+    try:
+        print(f"row subsets M={M} x={x_dtype} meta={meta_kind}", flush=True)
+        full = gpu.q4_linear(weight, x, x_dtype, engine.F32)
+        prefix = gpu.q4_linear_rows(weight, None, x, x_dtype, engine.F32, count=203)
+        gathered = gpu.q4_linear_rows(weight, ids, x, x_dtype, engine.F32)
+        gathered16 = gpu.q4_linear_rows(weight, ids, x, x_dtype, engine.F16)
+        with pytest.raises(engine.Mi355qError):
+            gpu.q4_linear_rows(weight, np.array([N], dtype=np.uint32), x, x_dtype, engine.F32)
+        with pytest.raises(engine.Mi355qError):
+            gpu.q4_linear_rows(weight, None, x, x_dtype, engine.F32, count=N + 1)
+    finally:
+        weight.destroy()
+    ref = oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_dtype, M)
+    assert prefix.shape == (M, 203) and gathered.shape == (M, ids.size)
+    assert q4_relative_error(full, ref) <= TOLERANCE
+    assert q4_relative_error(prefix, ref[:, :203]) <= TOLERANCE
+    assert q4_relative_error(gathered, ref[:, ids]) <= TOLERANCE
+    assert q4_relative_error(gathered16, ref[:, ids]) <= TOLERANCE
+    # the same arithmetic as the full linear; only the split of K over waves may differ
+    assert q4_relative_error(prefix, full[:, :203].astype(np.float64)) <= 1e-4
+    assert q4_relative_error(gathered, full[:, ids].astype(np.float64)) <= 1e-4
+
+
 def test_recorded_sequence_replays(engine, oracle, gpu):
     """mi355q_q4_sequence_record / mi355q_graph_launch: three calls (shared-x pair at M=1, an fp32
     activation that goes through the conversion kernel, an M=8 call that is cut in K slices and
