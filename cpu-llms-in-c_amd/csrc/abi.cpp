@@ -83,6 +83,8 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipStreamCreate(&ctx->stream);
     if (status == hipSuccess) status = hipEventCreate(&ctx->timer_start);
     if (status == hipSuccess) status = hipEventCreate(&ctx->timer_stop);
+    if (status == hipSuccess) status = hipMalloc((void **)&ctx->arrivals, kArrivalCounters * sizeof(uint32_t));
+    if (status == hipSuccess) status = hipMemset(ctx->arrivals, 0, kArrivalCounters * sizeof(uint32_t));
     if (status != hipSuccess) {
         int code = fail_hip(status, "context_create", error, error_capacity);
         mi355q_context_destroy(ctx);
@@ -103,6 +105,7 @@ void mi355q_context_destroy(mi355q_context *ctx)
         for (hipEvent_t event : *ctx->profile_events) (void)hipEventDestroy(event);
         delete ctx->profile_events;
     }
+    if (ctx->arrivals) (void)hipFree(ctx->arrivals);
     if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
     if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);

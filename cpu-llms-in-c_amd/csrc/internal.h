@@ -65,7 +65,13 @@ struct mi355q_context {
     // pointers and refuse to run once this has moved on
     uint64_t stage_generation;
     bool capturing;  // between hipStreamBeginCapture and EndCapture on `stream`
+    // arrival counters of K-sliced launches (one per workgroup column), zero between launches:
+    // the workgroup that arrives last adds the slices and puts its counter back to zero
+    uint32_t *arrivals;
 };
+namespace mi355q {
+constexpr uint32_t kArrivalCounters = 65536;
+}
 
 struct mi355q_q4_weight {
     mi355q_context *ctx;

@@ -21,8 +21,8 @@
 // wave reads its steps from there.  With several activation rows that copy is as
 // large as the weights a tile brings, so a workgroup then takes two tiles, long
 // rows are cut in slices over workgroups (fp32 partial sums, added in slice order
-// by a second small kernel), and a slice that still overflows LDS is walked in
-// chunks.
+// by whichever workgroup of the column finishes last), and a slice that still
+// overflows LDS is walked in chunks.
 #include "device_util.h"
 #include "internal.h"
 
@@ -55,6 +55,11 @@ struct StreamParams {
     // partial sums [slice][M][n_total] for the reduction kernel.
     uint32_t slices, slice_steps, chunk_steps;
     float *partials;
+    // Non-null: the workgroups of one column (blockIdx.x) count their arrivals here after
+    // writing their partial sums, and the one that arrives last adds all slices (in slice
+    // order) and writes y; null: a second kernel adds them.
+    uint32_t *arrivals;
+    uint32_t columns;  // workgroup columns with work (blockIdx.x below this)
     uint32_t n_total, n_first[kMaxTargets];
     int pair;
     int y_dtype, residual_dtype;
@@ -88,6 +93,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15u;
     const uint32_t kq = lane >> 4;
+    if (blockIdx.x >= p.columns) return;  // the grid is padded to a multiple of the XCD count
     uint32_t target = 0;
 #pragma unroll
     for (uint32_t t = 1; t < kMaxTargets; ++t)
@@ -299,7 +305,10 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 m = row >> 1;
             }
             if (p.slices > 1u) {
-                p.partials[((size_t)blockIdx.y * p.M + m) * p.n_total + p.n_first[slot_target] + n] = value;
+                // to L2 (agent scope), where the workgroup that adds the slices will read it
+                uint32_t *word = (uint32_t *)&p.partials[((size_t)blockIdx.y * p.M + m) * p.n_total +
+                                                         p.n_first[slot_target] + n];
+                __hip_atomic_store(word, __builtin_bit_cast(uint32_t, value), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 continue;
             }
             const size_t at = (size_t)m * N + n;
@@ -312,6 +321,58 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             if (p.ids != nullptr && p.ids[n] >= p.matrix_rows) value = 0.0f;  // no such row
             store_from_float(p.y[target], p.y_dtype, at, value);
         }
+    }
+    if (p.slices <= 1u || p.arrivals == nullptr) return;
+
+    // ---- K slices: the last workgroup of this column to get here adds them up.  Nobody waits
+    // for anybody: every workgroup publishes its partial sums, counts itself, and leaves unless
+    // it is the last.  The order of the additions is the slice order whoever does them.
+    // The workgroups of one column run on the same XCD (the grid's width is a multiple of the
+    // number of XCDs, over which workgroups are dealt round-robin in launch order), so they
+    // share one L2: the partial sums and the counter are written and read there (agent-scope
+    // accesses, which pass the per-CU cache), and a thread only has to know its stores have
+    // been acknowledged before the count goes up.  No device-wide cache write-back.
+    __shared__ uint32_t last_arrival;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this thread's stores have reached L2
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t before =
+            __hip_atomic_fetch_add(&p.arrivals[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_arrival = before + 1u == p.slices;
+        if (last_arrival)  // everyone has counted: ready for the next launch
+            __hip_atomic_store(&p.arrivals[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last_arrival) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    for (uint32_t e = threadIdx.x; e < TB * 64u * NJ; e += 64u * W) {
+        const uint32_t j = e % NJ, tb = (e / NJ) >> 6, l = (e / NJ) & 63u;
+        const uint32_t slot_target = p.fuse_silu ? tb / span_tiles : target;
+        const uint32_t tile = tile0 + tb % span_tiles;
+        const uint32_t n = tile * kTileRows + (l & 15u);
+        const uint32_t row = 4u * (l >> 4) + j;
+        if (tile >= NT || n >= N || row >= p.rows) continue;
+        if (p.fuse_silu && tb >= span_tiles) continue;  // the gate slot's thread does both
+        if (p.pair && (j & 1u)) continue;
+        const uint32_t m = p.pair ? row >> 1 : row;
+        auto total = [&](uint32_t column) {
+            float sum = 0.0f;
+            for (uint32_t s = 0; s < p.slices; ++s) {
+                const uint32_t *word = (const uint32_t *)&p.partials[((size_t)s * p.M + m) * p.n_total + column];
+                sum += __builtin_bit_cast(float, __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            }
+            return sum;
+        };
+        float value = total(p.n_first[slot_target] + n);
+        const size_t at = (size_t)m * N + n;
+        if (p.fuse_silu) {
+            store_from_float(p.y[0], p.y_dtype, at, silu_times(value, total(p.n_first[1] + n)));
+            continue;
+        }
+        if (p.residual[target])
+            value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
+        if (p.ids != nullptr && p.ids[n] >= p.matrix_rows) value = 0.0f;  // no such row
+        store_from_float(p.y[target], p.y_dtype, at, value);
     }
 }
 
@@ -389,10 +450,15 @@ static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
     else
         for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
     const size_t lds = stream_lds_bytes(MP, TB, W, p.chunk_steps);
-    const dim3 grid(blocks, p.slices);
-    if (p.meta_bf16)
-        return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, grid, dim3(64u * W), lds, p);
-    return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, grid, dim3(64u * W), lds, p);
+    StreamParams q = p;
+    q.columns = blocks;
+    // slices added in the kernel: the slices of one column must land on one XCD, which they do
+    // when the row of workgroups in front of each slice is a whole number of rounds over the XCDs
+    const uint32_t xcds = 8;
+    const dim3 grid(q.arrivals ? (blocks + xcds - 1) / xcds * xcds : blocks, q.slices);
+    if (q.meta_bf16)
+        return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, grid, dim3(64u * W), lds, q);
+    return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, grid, dim3(64u * W), lds, q);
 }
 
 template <int MP>
@@ -439,11 +505,18 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         // busy without queueing; more waves per workgroup when there are few tiles
         const uint32_t want = (16u * cus + NT_total - 1) / NT_total;
         shape.waves = want <= 2u ? 2 : want <= 5u ? 4 : 8;
+        if (NT_total <= cus + cus / 2u && T >= 96u) {
+            // few tiles with long rows (the 27B down projection): four K slices of pairs of
+            // tiles keep more loads in flight than eight waves on one tile each
+            shape.tb = 2;
+            shape.waves = 4;
+            slices = 4;
+        }
     } else {
         // every workgroup copies its activation rows from L2 into LDS: two tiles per
         // workgroup halve that traffic.  Matrices with few tiles and long rows are cut in
-        // slices (of 32 steps or more: the reduction launch costs about as much as
-        // 10 steps) until some 2.5 workgroups per compute unit exist.
+        // slices (of 32 steps or more: adding the slices costs about as much as a few
+        // steps) until some 2.5 workgroups per compute unit exist.
         shape.tb = NT_total >= cus ? 2 : 1;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
         slices = (5u * cus / 2u + groups / 2u) / groups;
@@ -462,7 +535,7 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         shape.waves = fw;
         if (fields >= 4 && fs >= 1) slices = (uint32_t)fs;
     }
-    choose_cuts(shape, T, mp == 1 ? 1u : slices);
+    choose_cuts(shape, T, slices);
     while (shape.waves > 2 && (uint32_t)shape.waves > shape.chunk_steps) shape.waves /= 2;
     return shape;
 }
@@ -540,6 +613,9 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
                                   error_capacity);
         if (status != MI355Q_OK) return status;
         p.partials = (float *)ctx->stage[4];
+        // grid.x of the launch: the workgroup columns that count arrivals
+        const uint32_t columns = a.fuse_silu ? (p.NT[0] + shape.tb / 2 - 1) / (shape.tb / 2) : block;
+        p.arrivals = columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
     }
     p.pair = pair;
     p.y_dtype = a.y_dtype;
@@ -548,7 +624,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.meta_bf16 = first.meta_kind == MI355Q_META_BF16_PLANES;
 
     const size_t lds = stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps);
-    if (lds > 64u * 1024u) {
+    if (lds + 64u > 64u * 1024u) {  // a few bytes of static LDS besides
         set_error(error, error_capacity, "q4 stream kernel: %zu bytes of LDS needed (K=%u, rows=%u)",
                   lds, first.K, rows);
         return MI355Q_ERROR_INVALID;
@@ -569,7 +645,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 stream kernel launch", error, error_capacity);
-    if (p.slices > 1u) {
+    if (p.slices > 1u && p.arrivals == nullptr) {
         launched = launch(ctx, q4_stream_reduce_kernel, dim3((p.n_total + 255u) / 256u, a.M), dim3(256), 0, p);
         if (launched != hipSuccess)
             return fail_hip(launched, "q4 stream reduce launch", error, error_capacity);
