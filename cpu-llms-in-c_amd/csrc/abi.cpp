@@ -85,6 +85,9 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipEventCreate(&ctx->timer_stop);
     if (status == hipSuccess) status = hipMalloc((void **)&ctx->arrivals, kArrivalCounters * sizeof(uint32_t));
     if (status == hipSuccess) status = hipMemset(ctx->arrivals, 0, kArrivalCounters * sizeof(uint32_t));
+    uint32_t xcds = 0;
+    if (status == hipSuccess) status = probe_columns_share_xcd(ctx, &ctx->columns_share_xcd, &xcds);
+    if (getenv("MI355Q_NO_ARRIVALS") != nullptr) ctx->columns_share_xcd = false;  // for comparisons
     if (status != hipSuccess) {
         int code = fail_hip(status, "context_create", error, error_capacity);
         mi355q_context_destroy(ctx);

@@ -68,6 +68,7 @@ struct mi355q_context {
     // arrival counters of K-sliced launches (one per workgroup column), zero between launches:
     // the workgroup that arrives last adds the slices and puts its counter back to zero
     uint32_t *arrivals;
+    bool columns_share_xcd;  // probed at creation; false switches that addition to a second kernel
 };
 namespace mi355q {
 constexpr uint32_t kArrivalCounters = 65536;
@@ -121,6 +122,9 @@ inline size_t dtype_bytes(int dtype) { return dtype == MI355Q_F32 ? 4u : 2u; }
 inline bool dtype_valid(int dtype) {
     return dtype == MI355Q_F16 || dtype == MI355Q_F32 || dtype == MI355Q_BF16;
 }
+
+// probe.hip
+hipError_t probe_columns_share_xcd(mi355q_context *ctx, bool *shared, uint32_t *xcds);
 
 // q4_layout.hip
 hipError_t q4_repack_launch(const uint32_t *codes_src, const uint16_t *meta_a,

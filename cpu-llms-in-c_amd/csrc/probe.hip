@@ -72,6 +72,59 @@ __global__ void __launch_bounds__(256) mfma_probe_kernel(float *out, int iterati
 
 using namespace mi355q;
 
+// Which XCD a workgroup runs on: the XCC_ID hardware register (bits 3:0).
+__global__ void xcd_probe_kernel(uint32_t *__restrict__ out)
+{
+    // s_getreg_b32 hwreg(HW_REG_XCC_ID, 0, 4): register 20, offset 0, four bits
+    const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20);
+    if (threadIdx.x == 0) out[blockIdx.y * gridDim.x + blockIdx.x] = xcd & 15u;
+}
+
+namespace mi355q {
+// Do the workgroups (x, 0), (x, 1), ... of a grid whose width is a multiple of eight run on
+// the same XCD?  (Workgroups are dealt round-robin over the XCDs in launch order, so they
+// should; the in-kernel addition of K slices relies on it and is switched off if not.)
+hipError_t probe_columns_share_xcd(mi355q_context *ctx, bool *shared, uint32_t *xcds)
+{
+    const uint32_t width = 40, height = 5;
+    uint32_t *out = nullptr, seen[width * height];
+    hipError_t status = hipMalloc((void **)&out, sizeof seen);
+    if (status != hipSuccess) return status;
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(width, height), dim3(64), 0, ctx->stream, out);
+    status = hipGetLastError();
+    if (status == hipSuccess)
+        status = hipMemcpyAsync(seen, out, sizeof seen, hipMemcpyDeviceToHost, ctx->stream);
+    if (status == hipSuccess) status = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(out);
+    if (status != hipSuccess) return status;
+    *shared = true;
+    uint32_t mask = 0;
+    for (uint32_t y = 0; y < height; ++y)
+        for (uint32_t x = 0; x < width; ++x) {
+            mask |= 1u << seen[y * width + x];
+            if (seen[y * width + x] != seen[x]) *shared = false;
+        }
+    *xcds = (uint32_t)__builtin_popcount(mask);
+    return hipSuccess;
+}
+}  // namespace mi355q
+
+extern "C" int mi355q_probe_xcd_columns(mi355q_context *ctx, int *columns_share_xcd, int *xcds,
+                                        char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || columns_share_xcd == nullptr || xcds == nullptr) {
+        set_error(error, error_capacity, "probe_xcd_columns: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    bool shared = false;
+    uint32_t count = 0;
+    MI355Q_HIP(mi355q::probe_columns_share_xcd(ctx, &shared, &count), "xcd probe");
+    *columns_share_xcd = shared ? 1 : 0;
+    *xcds = (int)count;
+    return MI355Q_OK;
+}
+
 extern "C" int mi355q_probe_mfma_rate(mi355q_context *ctx, int valu_per_mfma, int repeats,
                                       double *tflops, char *error, size_t error_capacity)
 {

@@ -615,7 +615,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         p.partials = (float *)ctx->stage[4];
         // grid.x of the launch: the workgroup columns that count arrivals
         const uint32_t columns = a.fuse_silu ? (p.NT[0] + shape.tb / 2 - 1) / (shape.tb / 2) : block;
-        p.arrivals = columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
+        p.arrivals = ctx->columns_share_xcd && columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
     }
     p.pair = pair;
     p.y_dtype = a.y_dtype;

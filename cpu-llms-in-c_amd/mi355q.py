@@ -75,6 +75,7 @@ SIGNATURES = {
     "mi355q_sym128_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _int, _u32, _c.POINTER(_vp), *_err]),
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
+    "mi355q_probe_xcd_columns": (_int, [_vp, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), *_err]),
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
@@ -260,6 +261,12 @@ class Context:
         _call(self.lib.mi355q_sym128_weight_prepare, self.handle, _ptr(records), N, K, record_order,
               flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
+
+    def probe_xcd_columns(self):
+        """(columns_share_xcd, xcds): see mi355q_probe_xcd_columns."""
+        shared, xcds = ctypes.c_int(), ctypes.c_int()
+        _call(self.lib.mi355q_probe_xcd_columns, self.handle, ctypes.byref(shared), ctypes.byref(xcds))
+        return bool(shared.value), xcds.value
 
     def q4_dequant_rows(self, weight: Q4Weight, rows, out_dtype: int = F32) -> np.ndarray:
         rows = np.ascontiguousarray(rows, dtype=np.uint32)

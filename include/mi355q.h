@@ -155,6 +155,15 @@ int mi355q_probe_read_bandwidth(mi355q_context *ctx, size_t bytes, size_t launch
                                 int repeats, int variant, double *gb_per_s,
                                 char *error, size_t error_capacity);
 
+/* Where workgroups run: *xcds = number of XCDs (accelerator dies) a small grid was spread
+ * over; *columns_share_xcd = 1 if the workgroups (x, 0), (x, 1), ... of a grid whose width
+ * is a multiple of eight all ran on the XCD of (x, 0).  The streaming kernel adds K slices
+ * inside the kernel only then (their partial sums meet in that XCD's L2); the context
+ * probes this once at creation and otherwise adds them with a second kernel.  No
+ * counterpart in the reference (single-die targets). */
+int mi355q_probe_xcd_columns(mi355q_context *ctx, int *columns_share_xcd, int *xcds,
+                             char *error, size_t error_capacity);
+
 /* Measured rate of the fp16 matrix instruction (v_mfma_f32_16x16x32_f16, fp32
  * accumulation) with every SIMD issuing independent ones from registers and
  * `valu_per_mfma` (0..4) packed-fp16 vector instructions between them — the mix of

@@ -287,6 +287,34 @@ def test_row_subsets(engine, oracle, gpu, M, x_dtype, meta_kind):
     assert q4_relative_error(gathered, full[:, ids].astype(np.float64)) <= 1e-4
 
 
+def test_slices_added_in_kernel_match_second_kernel(engine, oracle, gpu, monkeypatch):
+    """K slices are added by the last workgroup of a column to arrive, which needs the
+    workgroups of a column on one XCD (probed when a context is created).  The probe must
+    say so on this GPU, and a context created with the in-kernel addition switched off (a
+    second kernel adds the slices) must give the same bits: both add in slice order.
+    Repeated calls (the arrival counters return to zero) stay bitwise equal too."""
+    shared, xcds = gpu.probe_xcd_columns()
+    print(f"xcds={xcds} columns_share_xcd={shared}", flush=True)
+    assert shared and xcds >= 1
+    N, K, M = 320, 8704, 8
+    quants, meta_a, meta_b = engine.synth_q4_affine(41, 0.02, N, K, engine.META_BF16_PLANES)
+    x = make_x(engine, 42, M, K, engine.F16)
+    results = []
+    for off in (False, True):
+        if off:
+            monkeypatch.setenv("MI355Q_NO_ARRIVALS", "1")
+        ctx = engine.Context(0)
+        weight = ctx.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+        try:
+            results.append([ctx.q4_linear(weight, x, engine.F16, engine.F32) for _ in range(3)])
+        finally:
+            weight.destroy()
+    ref = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x, engine.F16, M)
+    assert q4_relative_error(results[0][0], ref) <= TOLERANCE
+    for y in results[0] + results[1]:
+        assert np.array_equal(y.view(np.uint32), results[0][0].view(np.uint32))
+
+
 def test_recorded_sequence_replays(engine, oracle, gpu):
     """mi355q_q4_sequence_record / mi355q_graph_launch: three calls (shared-x pair at M=1, an fp32
     activation that goes through the conversion kernel, an M=8 call that is cut in K slices and
