@@ -453,6 +453,12 @@ size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight)
     return weight ? weight->image_bytes : 0;
 }
 
+void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_t *K)
+{
+    if (N != nullptr) *N = weight ? weight->dev.N : 0;
+    if (K != nullptr) *K = weight ? weight->dev.K : 0;
+}
+
 int mi355q_q4_dequant_rows(mi355q_context *ctx, const mi355q_q4_weight *weight, const uint32_t *rows,
                            uint32_t count, void *out, int out_dtype, uint32_t flags, char *error,
                            size_t error_capacity)

@@ -809,7 +809,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     uint32_t best_splits = 1;
     double best_cost = 1e30;
     // the pipelined kernel addresses x with 32-bit byte offsets and whole 128-column steps
-    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * w.K * sizeof(_Float16) < (1ull << 32);
+    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * w.K * sizeof(_Float16) + 16384u < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
         if (v >= 6 && !pipe_ok) continue;
         const Variant &c = variants[v];

@@ -76,6 +76,18 @@ SIGNATURES = {
     "mi355q_q4_weight_destroy": (None, [_vp]),
     "mi355q_q4_weight_image_bytes": (_sz, [_vp]),
     "mi355q_probe_xcd_columns": (_int, [_vp, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), *_err]),
+    "mi355q_q4_weight_shape": (None, [_vp, ctypes.POINTER(_u32), ctypes.POINTER(_u32)]),
+    "mi355q_q38_image_open": (_int, [_vp, _vp, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p), *_err]),
+    "mi355q_q38_image_close": (None, [_vp]),
+    "mi355q_q38_image_kind": (_int, [_vp]),
+    "mi355q_q38_kind_name": (ctypes.c_char_p, [_int]),
+    "mi355q_q38_image_version": (_u32, [_vp]),
+    "mi355q_q38_image_layer_index": (_u32, [_vp]),
+    "mi355q_q38_image_linear_count": (ctypes.c_size_t, [_vp]),
+    "mi355q_q38_image_linear": (ctypes.c_void_p, [_vp, ctypes.c_size_t, ctypes.POINTER(ctypes.c_char_p)]),
+    "mi355q_q38_image_find": (ctypes.c_void_p, [_vp, ctypes.c_char_p]),
+    "mi355q_q38_layout_field": (_int, [_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_char_p),
+                                       ctypes.POINTER(_u32), ctypes.POINTER(_u32)]),
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
@@ -158,6 +170,42 @@ class Q4Weight:
         if self.handle:
             library().mi355q_q4_weight_destroy(self.handle)
             self.handle = None
+
+
+class Q38Image:
+    """An opened Qwen3.8 image file: its linears as prepared weights (owned by the image)."""
+
+    def __init__(self, context: "Context", handle):
+        lib = library()
+        self.context, self.handle = context, handle
+        self.kind = lib.mi355q_q38_kind_name(lib.mi355q_q38_image_kind(handle)).decode()
+        self.version = lib.mi355q_q38_image_version(handle)
+        self.layer_index = lib.mi355q_q38_image_layer_index(handle)
+        self.linears = {}
+        for index in range(lib.mi355q_q38_image_linear_count(handle)):
+            name = ctypes.c_char_p()
+            weight = ctypes.c_void_p(lib.mi355q_q38_image_linear(handle, index, ctypes.byref(name)))
+            N, K = _u32(), _u32()
+            lib.mi355q_q4_weight_shape(weight, ctypes.byref(N), ctypes.byref(K))
+            self.linears[name.value.decode()] = Q4Weight(context, weight, N.value, K.value)
+
+    def close(self):
+        if self.handle:
+            library().mi355q_q38_image_close(self.handle)
+            self.handle = None
+            for weight in self.linears.values():
+                weight.handle = None  # freed with the image
+
+
+def q38_layout_fields(kind: int) -> dict:
+    """{field name: (byte offset, size)} the loader reads from a header of that kind."""
+    lib, fields, index = library(), {}, 0
+    while True:
+        name, offset, size = ctypes.c_char_p(), _u32(), _u32()
+        if lib.mi355q_q38_layout_field(kind, index, ctypes.byref(name), ctypes.byref(offset), ctypes.byref(size)):
+            return fields
+        fields[name.value.decode()] = (offset.value, size.value)
+        index += 1
 
 
 class Context:
@@ -261,6 +309,13 @@ class Context:
         _call(self.lib.mi355q_sym128_weight_prepare, self.handle, _ptr(records), N, K, record_order,
               flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
+
+    def q38_image_open(self, image_bytes) -> Q38Image:
+        """Opens the bytes of a .q38delta / .q38att / .q38global / .q38mtp file."""
+        data = np.ascontiguousarray(np.frombuffer(image_bytes, dtype=np.uint8))
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_q38_image_open, self.handle, _ptr(data), data.size, ctypes.byref(out))
+        return Q38Image(self, out)
 
     def probe_xcd_columns(self):
         """(columns_share_xcd, xcds): see mi355q_probe_xcd_columns."""

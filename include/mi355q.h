@@ -206,6 +206,44 @@ int mi355q_sym128_weight_prepare(mi355q_context *ctx, const void *records,
 void mi355q_q4_weight_destroy(mi355q_q4_weight *weight);
 /* Bytes of the original image this weight stands for: N*K/2 + N*(K/64)*4. */
 size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight);
+/* Rows (outputs) and columns (inputs) of a prepared weight. */
+void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_t *K);
+
+/* ---- Qwen3.8 image files --------------------------------------------------------
+ * The reference's Apple M3 target keeps the model in four kinds of image file: a
+ * 4096-byte header, then per linear a code plane and a {fp16 scale, fp16 bias}
+ * metadata plane at the offsets the header names:
+ *   kind 0 "layer"     (.q38delta, magic "Q38M3Q4\0", versions 3 and 2 = MLP only):
+ *                      gate, up, down, delta_input, delta_output   (qwen38_m3_image.h:26-87)
+ *   kind 1 "attention" (.q38att, "Q38M3ATT"): gate, up, down, attention_input,
+ *                      attention_output                            (qwen38_m3_attention_image.h:21-70)
+ *   kind 2 "global"    (.q38global, "Q38M3GLB"): embedding, lm_head (qwen38_m3_global_image.h:15-44)
+ *   kind 3 "mtp"       (.q38mtp, "Q38M3MTP"): fc                    (qwen38_m3_mtp_image.h:16-45)
+ * mi355q_q38_image_open takes the bytes of one such file (read or mapped by the caller,
+ * who keeps them only for the duration of the call), checks magic, version, header size,
+ * group size, and that every linear's byte counts match its own row and column counts and
+ * lie inside the image (anything else: status 2, as the reference's loaders refuse a bad
+ * header, qwen38_m3.m:468-505, qwen38_m3_attention.m:138-160, qwen38_m3_decode.m:405-470),
+ * and prepares every linear as an ordinary Q4 weight owned by the image handle.  Unlike
+ * the reference it does not insist on the 27B dimensions or the source checksum.
+ * Replaces the header validation and newBufferWithBytesNoCopy mapping of those files. */
+typedef struct mi355q_q38_image mi355q_q38_image;
+int mi355q_q38_image_open(mi355q_context *ctx, const void *bytes, size_t size,
+                          mi355q_q38_image **out, char *error, size_t error_capacity);
+void mi355q_q38_image_close(mi355q_q38_image *image);
+int mi355q_q38_image_kind(const mi355q_q38_image *image);          /* 0..3 as above */
+const char *mi355q_q38_kind_name(int kind);
+uint32_t mi355q_q38_image_version(const mi355q_q38_image *image);
+uint32_t mi355q_q38_image_layer_index(const mi355q_q38_image *image); /* 0 for global / mtp */
+size_t mi355q_q38_image_linear_count(const mi355q_q38_image *image);
+/* The index-th linear (borrowed: valid until the image is closed) and its name. */
+const mi355q_q4_weight *mi355q_q38_image_linear(const mi355q_q38_image *image, size_t index,
+                                                const char **name);
+const mi355q_q4_weight *mi355q_q38_image_find(const mi355q_q38_image *image, const char *name);
+/* The header fields the loader reads, for checking against the reference's structs:
+ * field `index` of kind `kind` -> name, byte offset, size; status 2 past the end. */
+int mi355q_q38_layout_field(int kind, size_t index, const char **name, uint32_t *offset,
+                            uint32_t *bytes);
 
 /* out[i][k] = scale * q + bias of row rows[i] (fp32 multiply then add, rounded once to
  * out_dtype), [count][K]: the token-embedding lookup on a Q4 table,
