@@ -102,7 +102,7 @@ void mi355q_context_destroy(mi355q_context *ctx)
     if (ctx == nullptr) return;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    for (int slot = 0; slot < 5; ++slot)
+    for (int slot = 0; slot < 6; ++slot)
         if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
     if (ctx->profile_events) {
         for (hipEvent_t event : *ctx->profile_events) (void)hipEventDestroy(event);

@@ -58,9 +58,9 @@ struct mi355q_context {
     std::vector<hipEvent_t> *profile_events;
     size_t profile_used;
     // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16,
-    // 4 fp32 partial sums of a K-split GEMM
-    void *stage[5];
-    size_t stage_bytes[5];
+    // 4 fp32 partial sums of a K-split GEMM, 5 the high-nibble half of an affine-Q8 linear
+    void *stage[6];
+    size_t stage_bytes[6];
     // bumped whenever a staging buffer is reallocated: recorded graphs hold the old
     // pointers and refuse to run once this has moved on
     uint64_t stage_generation;

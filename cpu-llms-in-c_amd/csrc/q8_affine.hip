@@ -1,0 +1,195 @@
+// Affine Q8, group 64: w = scale * q + bias with 8-bit codes, u8 quants[N][K] and per
+// (row, 64-column group) scale and bias — the format of the reference's
+// minimax_h3_q8_gemm_bf16_meta (minimax_h3_attention.metal:594-676: element k of group g of
+// row n is byte (n * K/64 + g) * 64 + k; bf16 scales[N][K/64], biases[N][K/64]).
+//
+// A byte is two nibbles, q = 16 * hi + lo, so
+//     scale * q + bias = (16 * scale) * hi + bias   +   scale * lo
+// and an affine-Q8 matrix is the sum of two affine-Q4 matrices over the same columns: one
+// with the high nibbles, scale 16*scale (a power-of-two multiple: exact) and the bias, one
+// with the low nibbles, the scale, and bias 0.  prepare splits the bytes once on the GPU
+// into two ordinary stream-tiled Q4 weights; a linear is the first one into an fp32
+// buffer and the second one with that buffer as its residual.  Every Q4 kernel, shape
+// heuristic and epilogue serves as is; the bytes read are the Q8 image's plus a second copy
+// of the metadata (+6 %).  The bias sits with the high part so that the GEMM path, which
+// rounds a weight to fp16, rounds the same magnitude the reference's half(scale*q+bias) does.
+#include "internal.h"
+
+#include <cstring>
+#include <new>
+
+namespace mi355q {
+
+// One thread per eight codes: two output words (high and low nibbles in the Q4 source
+// layout, column k of eight at bits 4*(k%8)); threads of the first code word of a group
+// also write the group's two metadata pairs.
+__global__ void __launch_bounds__(256)
+q8_split_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ meta_a,
+                const uint16_t *__restrict__ meta_b, int meta_kind, uint32_t N, uint32_t K,
+                uint32_t *__restrict__ hi_codes, uint32_t *__restrict__ lo_codes,
+                uint16_t *__restrict__ hi_a, uint16_t *__restrict__ hi_b, uint16_t *__restrict__ lo_a,
+                uint16_t *__restrict__ lo_b)
+{
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t words = (uint64_t)N * (K / 8u);
+    if (index >= words) return;
+    const uint2 eight = ((const uint2 *)quants)[index];
+    uint32_t hi = 0, lo = 0;
+#pragma unroll
+    for (uint32_t c = 0; c < 8; ++c) {
+        const uint32_t byte = ((c < 4 ? eight.x : eight.y) >> (8u * (c & 3u))) & 255u;
+        hi |= (byte >> 4) << (4u * c);
+        lo |= (byte & 15u) << (4u * c);
+    }
+    hi_codes[index] = hi;
+    lo_codes[index] = lo;
+    if (index % 8u != 0) return;
+    const uint64_t block = index / 8u;  // (row, group)
+    if (meta_kind == MI355Q_META_F16_INTERLEAVED) {
+        const _Float16 scale = __builtin_bit_cast(_Float16, meta_a[2u * block]);
+        hi_a[2u * block] = __builtin_bit_cast(uint16_t, (_Float16)(scale * (_Float16)16.0f));
+        hi_a[2u * block + 1u] = meta_a[2u * block + 1u];
+        lo_a[2u * block] = meta_a[2u * block];
+        lo_a[2u * block + 1u] = 0;
+    } else {
+        const float scale = __builtin_bit_cast(float, (uint32_t)meta_a[block] << 16);
+        hi_a[block] = (uint16_t)(__builtin_bit_cast(uint32_t, scale * 16.0f) >> 16);  // exact
+        hi_b[block] = meta_b[block];
+        lo_a[block] = meta_a[block];
+        lo_b[block] = 0;
+    }
+}
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+struct mi355q_q8_weight {
+    mi355q_context *ctx;
+    mi355q_q4_weight *hi, *lo;
+    size_t image_bytes;
+};
+
+extern "C" void mi355q_q8_weight_destroy(mi355q_q8_weight *weight)
+{
+    if (weight == nullptr) return;
+    mi355q_q4_weight_destroy(weight->hi);
+    mi355q_q4_weight_destroy(weight->lo);
+    delete weight;
+}
+
+extern "C" size_t mi355q_q8_weight_image_bytes(const mi355q_q8_weight *weight)
+{
+    return weight ? weight->image_bytes : 0;
+}
+
+extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
+                                        const void *meta_b, uint32_t N, uint32_t K, int meta_kind,
+                                        uint32_t flags, mi355q_q8_weight **out, char *error,
+                                        size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    const bool planes = meta_kind == MI355Q_META_BF16_PLANES;
+    if (ctx == nullptr || out == nullptr || quants == nullptr || meta_a == nullptr ||
+        (planes && meta_b == nullptr) || (!planes && meta_kind != MI355Q_META_F16_INTERLEAVED)) {
+        set_error(error, error_capacity, "q8_weight_prepare: null argument or unknown metadata kind %d", meta_kind);
+        return MI355Q_ERROR_INVALID;
+    }
+    if (N == 0 || K == 0 || K % 64u != 0) {
+        set_error(error, error_capacity, "q8_weight_prepare: shape %u x %u (columns must be a non-zero multiple of 64)",
+                  N, K);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t groups = (size_t)N * (K / 64u);
+    const size_t code_bytes = (size_t)N * K, nibble_bytes = code_bytes / 2u;
+    const size_t plane_bytes = groups * 2u, meta_bytes = planes ? plane_bytes : 2u * plane_bytes;
+    auto aligned = [](size_t bytes) { return (bytes + 255u) & ~(size_t)255u; };
+    // source image (when it comes from the host) | hi codes | lo codes | hi meta a, b | lo meta a, b
+    const bool from_device = flags & MI355Q_SOURCE_DEVICE;
+    size_t at = 0;
+    const size_t at_quants = at;  at += from_device ? 0 : aligned(code_bytes);
+    const size_t at_meta_a = at;  at += from_device ? 0 : aligned(meta_bytes);
+    const size_t at_meta_b = at;  at += from_device || !planes ? 0 : aligned(meta_bytes);
+    const size_t at_hi = at;      at += aligned(nibble_bytes);
+    const size_t at_lo = at;      at += aligned(nibble_bytes);
+    size_t at_m[4];
+    for (int i = 0; i < 4; ++i) { at_m[i] = at; at += aligned(meta_bytes); }
+    char *scratch = nullptr;
+    MI355Q_HIP(hipMalloc((void **)&scratch, at), "q8 conversion buffer");
+    const void *d_quants = quants, *d_a = meta_a, *d_b = meta_b;
+    hipError_t status = hipSuccess;
+    if (!from_device) {
+        status = hipMemcpyAsync(scratch + at_quants, quants, code_bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (status == hipSuccess)
+            status = hipMemcpyAsync(scratch + at_meta_a, meta_a, meta_bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (status == hipSuccess && planes)
+            status = hipMemcpyAsync(scratch + at_meta_b, meta_b, meta_bytes, hipMemcpyHostToDevice, ctx->stream);
+        d_quants = scratch + at_quants;
+        d_a = scratch + at_meta_a;
+        d_b = planes ? scratch + at_meta_b : nullptr;
+    }
+    if (status == hipSuccess) {
+        const uint64_t words = (uint64_t)N * (K / 8u);
+        hipLaunchKernelGGL(q8_split_kernel, dim3((uint32_t)((words + 255u) / 256u)), dim3(256), 0, ctx->stream,
+                           (const uint8_t *)d_quants, (const uint16_t *)d_a, (const uint16_t *)d_b, meta_kind, N, K,
+                           (uint32_t *)(scratch + at_hi), (uint32_t *)(scratch + at_lo),
+                           (uint16_t *)(scratch + at_m[0]), (uint16_t *)(scratch + at_m[1]),
+                           (uint16_t *)(scratch + at_m[2]), (uint16_t *)(scratch + at_m[3]));
+        status = hipGetLastError();
+    }
+    int code = MI355Q_OK;
+    mi355q_q4_weight *hi = nullptr, *lo = nullptr;
+    if (status != hipSuccess) code = fail_hip(status, "q8 split", error, error_capacity);
+    if (code == MI355Q_OK)  // stream order: the re-tiling kernels run after the split
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_hi, scratch + at_m[0], planes ? scratch + at_m[1] : nullptr,
+                                        N, K, meta_kind, MI355Q_SOURCE_DEVICE, &hi, error, error_capacity);
+    if (code == MI355Q_OK)
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_lo, scratch + at_m[2], planes ? scratch + at_m[3] : nullptr,
+                                        N, K, meta_kind, MI355Q_SOURCE_DEVICE, &lo, error, error_capacity);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(scratch);
+    mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
+    if (code == MI355Q_OK && weight == nullptr) {
+        set_error(error, error_capacity, "q8_weight_prepare: out of host memory");
+        code = MI355Q_ERROR_RUNTIME;
+    }
+    if (code != MI355Q_OK) {
+        mi355q_q4_weight_destroy(hi);
+        mi355q_q4_weight_destroy(lo);
+        return code;
+    }
+    weight->ctx = ctx;
+    weight->hi = hi;
+    weight->lo = lo;
+    weight->image_bytes = code_bytes + groups * 4u;
+    *out = weight;
+    return MI355Q_OK;
+}
+
+extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *weight, const void *x, int x_dtype,
+                                uint32_t M, void *y, int y_dtype, const void *residual, int residual_dtype,
+                                uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || x == nullptr || y == nullptr || M == 0) {
+        set_error(error, error_capacity, "q8_linear: null argument or M = 0");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "q8_linear: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    uint32_t N = 0;
+    mi355q_q4_weight_shape(weight->hi, &N, nullptr);
+    // the high part (+ the caller's residual) into fp32, then the low part on top of it
+    int status = ensure_stage(ctx, 5, (size_t)M * N * sizeof(float), error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    void *partial = ctx->stage[5];
+    const uint32_t keep = flags & (MI355Q_X_DEVICE | MI355Q_ASYNC);
+    status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, residual, residual_dtype,
+                              keep | MI355Q_Y_DEVICE | (flags & (MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
+                              error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    return mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, y, y_dtype, partial, MI355Q_F32,
+                            keep | (flags & MI355Q_Y_DEVICE) | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+}

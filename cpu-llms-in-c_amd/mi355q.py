@@ -88,6 +88,10 @@ SIGNATURES = {
     "mi355q_q38_image_find": (ctypes.c_void_p, [_vp, ctypes.c_char_p]),
     "mi355q_q38_layout_field": (_int, [_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_char_p),
                                        ctypes.POINTER(_u32), ctypes.POINTER(_u32)]),
+    "mi355q_q8_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32, ctypes.POINTER(ctypes.c_void_p), *_err]),
+    "mi355q_q8_weight_destroy": (None, [_vp]),
+    "mi355q_q8_weight_image_bytes": (ctypes.c_size_t, [_vp]),
+    "mi355q_q8_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
@@ -309,6 +313,25 @@ class Context:
         _call(self.lib.mi355q_sym128_weight_prepare, self.handle, _ptr(records), N, K, record_order,
               flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
+
+    # ---- affine Q8 (two Q4 weights) ----
+    def q8_prepare(self, quants, meta_a, meta_b, N: int, K: int, meta_kind: int):
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_q8_weight_prepare, self.handle, _ptr(quants), _ptr(meta_a), _ptr(meta_b), N, K,
+              meta_kind, 0, ctypes.byref(out))
+        return out
+
+    def q8_destroy(self, weight):
+        self.lib.mi355q_q8_weight_destroy(weight)
+
+    def q8_linear(self, weight, N: int, x: np.ndarray, x_dtype: int, y_dtype: int = F32,
+                  residual: np.ndarray | None = None, residual_dtype: int = F32) -> np.ndarray:
+        x = np.ascontiguousarray(x)
+        M = x.shape[0]
+        y = np.empty((M, N), dtype=_NP_DTYPE[y_dtype])
+        _call(self.lib.mi355q_q8_linear, self.handle, weight, _ptr(x), x_dtype, M, _ptr(y), y_dtype,
+              _ptr(residual), residual_dtype, 0)
+        return y
 
     def q38_image_open(self, image_bytes) -> Q38Image:
         """Opens the bytes of a .q38delta / .q38att / .q38global / .q38mtp file."""

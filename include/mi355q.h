@@ -209,6 +209,26 @@ size_t mi355q_q4_weight_image_bytes(const mi355q_q4_weight *weight);
 /* Rows (outputs) and columns (inputs) of a prepared weight. */
 void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_t *K);
 
+/* ---- affine Q8, group 64 ---------------------------------------------------------
+ * w = scale * q + bias with one 8-bit code per byte, quants[N][K] (element k of group g of
+ * row n at byte (n * K/64 + g) * 64 + k), metadata as for Q4 (bf16 planes scales[N][K/64],
+ * biases[N][K/64], or fp16 pairs): the projection format of minimax_h3_q8_gemm_bf16_meta
+ * (minimax_h3_attention.metal:594-676).  prepare splits the codes into nibbles once:
+ * scale*q + bias = (16*scale)*hi + bias + scale*lo, two ordinary Q4 weights, and
+ * mi355q_q8_linear runs the two Q4 linears back to back (the second adds to the first in
+ * fp32); arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the
+ * GEMM path rounds each part to fp16 as the reference rounds half(scale*q + bias). */
+typedef struct mi355q_q8_weight mi355q_q8_weight;
+int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
+                             const void *meta_b, uint32_t N, uint32_t K, int meta_kind,
+                             uint32_t flags, mi355q_q8_weight **out,
+                             char *error, size_t error_capacity);
+void mi355q_q8_weight_destroy(mi355q_q8_weight *weight);
+size_t mi355q_q8_weight_image_bytes(const mi355q_q8_weight *weight); /* N*K + N*(K/64)*4 */
+int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *weight, const void *x,
+                     int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,
+                     int residual_dtype, uint32_t flags, char *error, size_t error_capacity);
+
 /* ---- Qwen3.8 image files --------------------------------------------------------
  * The reference's Apple M3 target keeps the model in four kinds of image file: a
  * 4096-byte header, then per linear a code plane and a {fp16 scale, fp16 bias}

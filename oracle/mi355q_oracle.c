@@ -92,6 +92,7 @@ typedef struct {
     const uint16_t *meta_b;
     int meta_kind;
     size_t groups;
+    unsigned bits; /* 4: two codes per byte; 8: one (the affine Q8 of minimax_h3_attention.metal:594-676) */
 } q4_matrix;
 
 static void q4_group_meta(const q4_matrix *w, size_t block, float *scale, float *bias)
@@ -111,6 +112,8 @@ static unsigned q4_code(const q4_matrix *w, size_t block, size_t j)
 {
     /* byte j/2 of the block's 32; even j in the low nibble:
      * qwen38_m3.m:113-115, real_gemm.c:36-37 */
+    if (w->bits == 8u) /* codes[k] of the block's 64: minimax_h3_attention.metal:631-634 */
+        return w->quants[block * 64u + j];
     uint8_t byte = w->quants[block * 32u + (j >> 1)];
     return (j & 1u) ? (unsigned)(byte >> 4) : (unsigned)(byte & 15u);
 }
@@ -187,7 +190,7 @@ int orc_q4_dequantize_row(const uint8_t *quants, const void *meta_a, const void 
 {
     if (!quants || !meta_a || !output || columns == 0 || columns % 64u != 0) return 1;
     q4_matrix w = {quants, (const uint16_t *)meta_a, (const uint16_t *)meta_b, meta_kind,
-                   columns / 64u};
+                   columns / 64u, 4u};
     for (size_t g = 0; g < w.groups; ++g) {
         size_t block = (size_t)row * w.groups + g;
         float scale, bias;
@@ -209,7 +212,7 @@ int orc_q4_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
     if (meta_kind == ORC_META_BF16_PLANES && !meta_b) return 2;
     if (row_end > N || row_begin > row_end) return 2;
     q4_matrix w = {quants, (const uint16_t *)meta_a, (const uint16_t *)meta_b,
-                   meta_kind, K / 64u};
+                   meta_kind, K / 64u, 4u};
 #ifdef _OPENMP
     int use = threads > 0 ? threads : omp_get_max_threads();
 #else
@@ -233,17 +236,41 @@ int orc_q4_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
     return 0;
 }
 
+/* Affine Q8, group 64 (u8 codes, the same metadata kinds): w = scale * q + bias with q in
+ * 0..255.  ORC_W_ROUND_F16 is the reference kernel's half(scale * float(q) + bias)
+ * (minimax_h3_attention.metal:628-634); the reference then accumulates a group in half
+ * and groups in fp32 (:640-667), which this does not imitate: sequential fp32 or double. */
+int orc_q8_affine_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
+                         int meta_kind, uint32_t N, uint32_t K,
+                         const void *x, int x_kind, uint32_t M,
+                         int weight_rounding, int accumulate, double *y)
+{
+    if (!quants || !meta_a || !x || !y || K == 0u || K % 64u != 0u) return 2;
+    if (meta_kind == ORC_META_BF16_PLANES && !meta_b) return 2;
+    q4_matrix w = {quants, (const uint16_t *)meta_a, (const uint16_t *)meta_b, meta_kind, K / 64u, 8u};
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t row = 0; row < (int64_t)N; ++row)
+        for (uint32_t m = 0; m < M; ++m)
+            y[(size_t)m * N + (size_t)row] =
+                accumulate == ORC_ACC_F64
+                    ? q4_row_f64(&w, (size_t)row, x, x_kind, (size_t)m * K, weight_rounding)
+                    : (double)q4_row_seq(&w, (size_t)row, x, x_kind, (size_t)m * K, weight_rounding);
+    return 0;
+}
+
 float orc_q4_dot_f16x_seq(const uint8_t *quants, const uint16_t *meta_interleaved,
                           const uint16_t *x_f16, size_t row, size_t groups)
 {
-    q4_matrix w = {quants, meta_interleaved, NULL, ORC_META_F16_INTERLEAVED, groups};
+    q4_matrix w = {quants, meta_interleaved, NULL, ORC_META_F16_INTERLEAVED, groups, 4u};
     return q4_row_seq(&w, row, x_f16, ORC_X_F16, 0, ORC_W_EXACT);
 }
 
 float orc_q4_dot_f32x_seq(const uint8_t *quants, const uint16_t *meta_interleaved,
                           const float *x, size_t row, size_t groups)
 {
-    q4_matrix w = {quants, meta_interleaved, NULL, ORC_META_F16_INTERLEAVED, groups};
+    q4_matrix w = {quants, meta_interleaved, NULL, ORC_META_F16_INTERLEAVED, groups, 4u};
     return q4_row_seq(&w, row, x, ORC_X_F32, 0, ORC_W_EXACT);
 }
 

@@ -84,6 +84,14 @@ int orc_q4_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
                   uint32_t row_begin, uint32_t row_end,
                   double *y, int threads);
 
+/* The same for affine Q8, group 64 (one code per byte, quants[N][K]): the format of
+ * minimax_h3_q8_gemm_bf16_meta (minimax_h3_attention.metal:594-676).  All rows.
+ * Pinned by tests/test_oracle_q4.py against a numpy float64 product. */
+int orc_q8_affine_linear(const uint8_t *quants, const void *meta_a, const void *meta_b,
+                         int meta_kind, uint32_t N, uint32_t K,
+                         const void *x, int x_kind, uint32_t M,
+                         int weight_rounding, int accumulate, double *y);
+
 /* Single-row convenience forms of the same thing. */
 float orc_q4_dot_f16x_seq(const uint8_t *quants, const uint16_t *meta_interleaved,
                           const uint16_t *x_f16, size_t row, size_t groups);

@@ -45,6 +45,8 @@ def lib() -> ctypes.CDLL:
         l.orc_q4_linear.restype = _int
         l.orc_q4_linear.argtypes = [_vp, _vp, _vp, _int, _u32, _u32, _vp, _int, _u32, _int,
                                     _int, _u32, _u32, _vp, _int]
+        l.orc_q8_affine_linear.restype = _int
+        l.orc_q8_affine_linear.argtypes = [_vp, _vp, _vp, _int, _u32, _u32, _vp, _int, _u32, _int, _int, _vp]
         l.orc_q4_dot_f16x_seq.restype = _c.c_float
         l.orc_q4_dot_f16x_seq.argtypes = [_vp, _vp, _vp, _sz, _sz]
         l.orc_q4_dot_f32x_seq.restype = _c.c_float
@@ -116,6 +118,18 @@ def q4_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_kind, M,
                                  threads)
     if status != 0:
         raise ValueError(f"orc_q4_linear status {status}")
+    return y
+
+
+def q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_kind, M,
+                     weight_rounding=W_EXACT, accumulate=ACC_F64):
+    """Affine Q8 g64 (u8 quants [N][K]): y [M][N] float64."""
+    x = np.ascontiguousarray(x)
+    y = np.zeros((M, N), dtype=np.float64)
+    status = lib().orc_q8_affine_linear(_p(quants), _p(meta_a), _p(meta_b), meta_kind, N, K, _p(x), x_kind, M,
+                                        weight_rounding, accumulate, _p(y))
+    if status != 0:
+        raise ValueError(f"orc_q8_affine_linear status {status}")
     return y
 
 

@@ -1,0 +1,70 @@
+"""GPU parity of the affine-Q8 g64 linear (two Q4 weights, mi355q_q8_linear) against the oracle.
+
+Format and reference arithmetic: minimax_h3_q8_gemm_bf16_meta (minimax_h3_attention.metal:594-676),
+u8 quants[N][K], bf16 scales/biases [N][K/64], weight = scale * q + bias.
+Gate for M <= 16 (weights kept exact): max_i |y_i - ref_i| / max(|ref_i|, 1e-2*rms(ref)) <= 1e-3
+against the exact weight with double accumulation.  The GEMM path (M > 16) rounds the two
+nibble halves of a weight to fp16 separately, the reference rounds half(scale*q+bias) once:
+both are within fp16 rounding of the exact weight but not of each other, so the gate there is
+the distance to the exact-weight result, max_i |y_i - ref_i| <= 2e-3 * rms(ref) (the bound the
+Q4 GEMM tests report for fp16-rounded weights), with the reference's own rounding held to the
+same bound for comparison."""
+import numpy as np
+import pytest
+
+from conftest import bf16_bits, q4_relative_error
+
+pytestmark = pytest.mark.gpu
+
+
+def make_q8(engine, seed, N, K, meta_kind):
+    """Seeded N(0, 0.02) weights, min/max affine 8-bit per group of 64 (metadata rounded first)."""
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((N, K // 64, 64)) * 0.02).astype(np.float32)
+    lo, hi = w.min(axis=2), w.max(axis=2)
+    scale = np.where(hi > lo, (hi - lo) / 255.0, 1.0).astype(np.float32)
+    if meta_kind == engine.META_BF16_PLANES:
+        scale_bits, bias_bits = bf16_bits(scale), bf16_bits(lo)
+        scale_r = (scale_bits.astype(np.uint32) << 16).view(np.float32)
+        bias_r = (bias_bits.astype(np.uint32) << 16).view(np.float32)
+        meta_a, meta_b = scale_bits.reshape(-1), bias_bits.reshape(-1)
+    else:
+        scale_r, bias_r = scale.astype(np.float16).astype(np.float32), lo.astype(np.float16).astype(np.float32)
+        meta_a = np.stack([scale_r.astype(np.float16).view(np.uint16), bias_r.astype(np.float16).view(np.uint16)],
+                          axis=-1).reshape(-1)
+        meta_b = None
+    q = np.clip(np.rint((w - bias_r[..., None]) / scale_r[..., None]), 0, 255).astype(np.uint8)
+    return np.ascontiguousarray(q.reshape(-1)), np.ascontiguousarray(meta_a), meta_b
+
+
+@pytest.mark.parametrize("N,K,M,meta", [(100, 192, 1, "META_BF16_PLANES"), (256, 1024, 1, "META_F16_INTERLEAVED"),
+                                        (1024, 3072, 4, "META_BF16_PLANES"), (320, 8704, 8, "META_BF16_PLANES"),
+                                        (528, 1536, 64, "META_BF16_PLANES"), (1088, 640, 200, "META_F16_INTERLEAVED")])
+def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
+    meta_kind = getattr(engine, meta)
+    quants, meta_a, meta_b = make_q8(engine, 3, N, K, meta_kind)
+    x = np.stack([engine.synth_normal_f32(70 + m, 1.0, K) for m in range(M)]).astype(np.float16)
+    residual = engine.synth_normal_f32(99, 1.0, M * N).reshape(M, N)
+    weight = gpu.q8_prepare(quants, meta_a, meta_b, N, K, meta_kind)
+    try:
+        print(f"q8 affine N={N} K={K} M={M} meta={meta}", flush=True)
+        assert engine.library().mi355q_q8_weight_image_bytes(weight) == N * K + N * (K // 64) * 4
+        y = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
+        y16 = gpu.q8_linear(weight, N, x, engine.F16, engine.F16)
+        with_residual = gpu.q8_linear(weight, N, x, engine.F16, engine.F32, residual, engine.F32)
+    finally:
+        gpu.q8_destroy(weight)
+    exact = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, engine.F16, M)
+    if M <= 16:
+        assert q4_relative_error(y, exact) <= 1e-3
+        assert q4_relative_error(y16, exact) <= 1e-3
+        assert q4_relative_error(with_residual, exact + residual) <= 1e-3
+    else:
+        rounded = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, engine.F16, M,
+                                          weight_rounding=oracle.W_ROUND_F16)
+        rms = np.sqrt(np.mean(exact * exact, axis=1, keepdims=True))
+        ours = float(np.max(np.abs(y - exact) / rms))
+        theirs = float(np.max(np.abs(rounded - exact) / rms))
+        print(f"distance to exact weights / rms: this library {ours:.2e}, half(scale*q+bias) {theirs:.2e}", flush=True)
+        assert ours <= 2e-3 and theirs <= 2e-3
+        assert float(np.max(np.abs(with_residual - (exact + residual)) / rms)) <= 2e-3

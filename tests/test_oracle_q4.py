@@ -212,3 +212,33 @@ def test_dequantize_row_equals_numpy_float32(oracle, meta_kind):
     rows = [0, 7, 22, 7]
     got = oracle.q4_dequantize_rows(quants, meta_a, meta_b, meta_kind, K, rows)
     assert np.array_equal(got.view(np.uint32), expect[rows].view(np.uint32))
+
+
+def test_q8_affine_matches_numpy_float64(oracle):
+    """orc_q8_affine_linear (u8 codes, one per byte) against a float64 matrix product on the codes
+    read straight from the byte array; a single hot code at eight (row, k) positions isolates the
+    index mapping (byte (n*K/64 + g)*64 + k, minimax_h3_attention.metal:631-634)."""
+    rng = np.random.default_rng(11)
+    N, K, M = 37, 320, 3
+    quants = rng.integers(0, 256, size=N * K, dtype=np.uint8)
+    scales = (rng.random(N * (K // 64), dtype=np.float32) * 0.01 + 0.001).astype(np.float16)
+    biases = (rng.standard_normal(N * (K // 64)).astype(np.float32) * 0.1).astype(np.float16)
+    meta = np.stack([scales.view(np.uint16), biases.view(np.uint16)], axis=-1).reshape(-1)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    w = (scales.astype(np.float64).reshape(N, -1, 1) * quants.reshape(N, -1, 64).astype(np.float64)
+         + biases.astype(np.float64).reshape(N, -1, 1)).reshape(N, K)
+    expect = x.astype(np.float64) @ w.T
+    got = oracle.q8_affine_linear(quants, meta, None, oracle.META_F16_INTERLEAVED, N, K, x, oracle.X_F16, M)
+    assert np.max(np.abs(got - expect)) <= 1e-9 * np.max(np.abs(expect))
+    for n, k in [(0, 0), (0, 63), (0, 64), (5, 131), (36, 319), (17, 1), (20, 200), (36, 0)]:
+        hot = np.zeros(N * K, dtype=np.uint8)
+        hot[n * K + k] = 200
+        one = np.stack([np.float16(1.0).view(np.uint16), np.float16(0.0).view(np.uint16)])
+        meta_one = np.tile(one, N * (K // 64))
+        y = oracle.q8_affine_linear(hot, meta_one, None, oracle.META_F16_INTERLEAVED, N, K, x, oracle.X_F16, M)
+        expect_hot = np.zeros((M, N))
+        expect_hot[:, n] = 200.0 * x[:, k].astype(np.float64)
+        assert np.array_equal(y, expect_hot)
+    seq = oracle.q8_affine_linear(quants, meta, None, oracle.META_F16_INTERLEAVED, N, K, x, oracle.X_F16, M,
+                                  accumulate=oracle.ACC_F32_SEQUENTIAL)
+    assert np.max(np.abs(seq - expect)) <= 1e-4 * np.max(np.abs(expect))
