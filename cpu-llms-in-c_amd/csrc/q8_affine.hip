@@ -13,6 +13,7 @@
 // heuristic and epilogue serves as is; the bytes read are the Q8 image's plus a second copy
 // of the metadata (+6 %).  The bias sits with the high part so that the GEMM path, which
 // rounds a weight to fp16, rounds the same magnitude the reference's half(scale*q+bias) does.
+#include "device_util.h"
 #include "internal.h"
 
 #include <cstring>
@@ -60,6 +61,57 @@ q8_split_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__
     }
 }
 
+// Q8 rows: per output row an fp32 scale and K signed bytes, w = scale * v
+// (the MMO_Q8_ROW tensors of minimindo_thinker.c:84-86,112-122 and the Q8 payload of
+// minimindo_audio_encoder.c:90,216-217).  v + 128 = 16 * hi + lo gives two Q4 weights with
+// the integer metadata {16, -128} and {1, 0} (exact in bf16), whose sum is the exact integer
+// dot product; the row's fp32 scale multiplies the finished sum, as the reference does.
+// One thread per eight codes.
+__global__ void __launch_bounds__(256)
+q8rows_split_kernel(const uint8_t *__restrict__ records, uint32_t N, uint32_t K,
+                    uint32_t *__restrict__ hi_codes, uint32_t *__restrict__ lo_codes,
+                    uint16_t *__restrict__ hi_a, uint16_t *__restrict__ hi_b, uint16_t *__restrict__ lo_a,
+                    uint16_t *__restrict__ lo_b, float *__restrict__ row_scale)
+{
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t words_per_row = K / 8u;
+    if (index >= (uint64_t)N * words_per_row) return;
+    const uint32_t row = (uint32_t)(index / words_per_row), word = (uint32_t)(index % words_per_row);
+    const uint8_t *record = records + (size_t)row * (4u + K);  // only byte-aligned
+    uint32_t hi = 0, lo = 0;
+#pragma unroll
+    for (uint32_t c = 0; c < 8; ++c) {
+        const uint32_t code = (uint32_t)(uint8_t)(record[4u + 8u * word + c] + 128u);  // v + 128 in 0..255
+        hi |= (code >> 4) << (4u * c);
+        lo |= (code & 15u) << (4u * c);
+    }
+    hi_codes[index] = hi;
+    lo_codes[index] = lo;
+    if (word % 8u == 0) {  // first word of a 64-column group
+        const uint64_t block = (uint64_t)row * (K / 64u) + word / 8u;
+        hi_a[block] = 0x4180;  // bf16 16
+        hi_b[block] = 0xc300;  // bf16 -128
+        lo_a[block] = 0x3f80;  // bf16 1
+        lo_b[block] = 0;
+    }
+    if (word == 0)
+        row_scale[row] = __builtin_bit_cast(float, (uint32_t)record[0] | (uint32_t)record[1] << 8 |
+                                                       (uint32_t)record[2] << 16 | (uint32_t)record[3] << 24);
+}
+
+// y[m][n] = sum[m][n] * scale[n] (+ residual), one thread per element
+__global__ void __launch_bounds__(256)
+q8rows_finish_kernel(const float *__restrict__ sum, const float *__restrict__ scale, const void *residual,
+                     int residual_dtype, int residual_is_bias, void *y, int y_dtype, uint32_t M, uint32_t N)
+{
+    const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= (size_t)M * N) return;
+    const uint32_t n = (uint32_t)(at % N);
+    float value = __fmul_rn(sum[at], scale[n]);
+    if (residual) value += load_as_float(residual, residual_dtype, residual_is_bias ? n : at);
+    store_from_float(y, y_dtype, at, value);
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -67,6 +119,7 @@ using namespace mi355q;
 struct mi355q_q8_weight {
     mi355q_context *ctx;
     mi355q_q4_weight *hi, *lo;
+    float *row_scale;  // Q8 rows: the fp32 scale of every output row (device); else null
     size_t image_bytes;
 };
 
@@ -75,6 +128,7 @@ extern "C" void mi355q_q8_weight_destroy(mi355q_q8_weight *weight)
     if (weight == nullptr) return;
     mi355q_q4_weight_destroy(weight->hi);
     mi355q_q4_weight_destroy(weight->lo);
+    if (weight->row_scale) (void)hipFree(weight->row_scale);
     delete weight;
 }
 
@@ -162,7 +216,80 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
     weight->ctx = ctx;
     weight->hi = hi;
     weight->lo = lo;
+    weight->row_scale = nullptr;
     weight->image_bytes = code_bytes + groups * 4u;
+    *out = weight;
+    return MI355Q_OK;
+}
+
+extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *records, uint32_t N, uint32_t K,
+                                            uint32_t flags, mi355q_q8_weight **out, char *error,
+                                            size_t error_capacity)
+{
+    if (out != nullptr) *out = nullptr;
+    if (ctx == nullptr || out == nullptr || records == nullptr) {
+        set_error(error, error_capacity, "q8rows_weight_prepare: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (N == 0 || K == 0 || K % 64u != 0) {
+        set_error(error, error_capacity,
+                  "q8rows_weight_prepare: shape %u x %u (columns must be a non-zero multiple of 64)", N, K);
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const size_t record_bytes = (size_t)N * (4u + K), nibble_bytes = (size_t)N * K / 2u;
+    const size_t plane_bytes = (size_t)N * (K / 64u) * 2u;
+    auto aligned = [](size_t bytes) { return (bytes + 255u) & ~(size_t)255u; };
+    const bool from_device = flags & MI355Q_SOURCE_DEVICE;
+    size_t at = from_device ? 0 : aligned(record_bytes);
+    const size_t at_hi = at;  at += aligned(nibble_bytes);
+    const size_t at_lo = at;  at += aligned(nibble_bytes);
+    size_t at_m[4];
+    for (int i = 0; i < 4; ++i) { at_m[i] = at; at += aligned(plane_bytes); }
+    char *scratch = nullptr;
+    float *row_scale = nullptr;
+    MI355Q_HIP(hipMalloc((void **)&scratch, at), "q8 rows conversion buffer");
+    hipError_t status = hipMalloc((void **)&row_scale, (size_t)N * sizeof(float));
+    const uint8_t *source = (const uint8_t *)records;
+    if (status == hipSuccess && !from_device) {
+        status = hipMemcpyAsync(scratch, records, record_bytes, hipMemcpyHostToDevice, ctx->stream);
+        source = (const uint8_t *)scratch;
+    }
+    if (status == hipSuccess) {
+        const uint64_t words = (uint64_t)N * (K / 8u);
+        hipLaunchKernelGGL(q8rows_split_kernel, dim3((uint32_t)((words + 255u) / 256u)), dim3(256), 0, ctx->stream,
+                           source, N, K, (uint32_t *)(scratch + at_hi), (uint32_t *)(scratch + at_lo),
+                           (uint16_t *)(scratch + at_m[0]), (uint16_t *)(scratch + at_m[1]),
+                           (uint16_t *)(scratch + at_m[2]), (uint16_t *)(scratch + at_m[3]), row_scale);
+        status = hipGetLastError();
+    }
+    int code = MI355Q_OK;
+    mi355q_q4_weight *hi = nullptr, *lo = nullptr;
+    if (status != hipSuccess) code = fail_hip(status, "q8 rows split", error, error_capacity);
+    if (code == MI355Q_OK)
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_hi, scratch + at_m[0], scratch + at_m[1], N, K,
+                                        MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &hi, error, error_capacity);
+    if (code == MI355Q_OK)
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_lo, scratch + at_m[2], scratch + at_m[3], N, K,
+                                        MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &lo, error, error_capacity);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(scratch);
+    mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
+    if (code == MI355Q_OK && weight == nullptr) {
+        set_error(error, error_capacity, "q8rows_weight_prepare: out of host memory");
+        code = MI355Q_ERROR_RUNTIME;
+    }
+    if (code != MI355Q_OK) {
+        mi355q_q4_weight_destroy(hi);
+        mi355q_q4_weight_destroy(lo);
+        if (row_scale) (void)hipFree(row_scale);
+        return code;
+    }
+    weight->ctx = ctx;
+    weight->hi = hi;
+    weight->lo = lo;
+    weight->row_scale = row_scale;
+    weight->image_bytes = record_bytes;
     *out = weight;
     return MI355Q_OK;
 }
@@ -181,15 +308,61 @@ extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *wei
     }
     uint32_t N = 0;
     mi355q_q4_weight_shape(weight->hi, &N, nullptr);
-    // the high part (+ the caller's residual) into fp32, then the low part on top of it
-    int status = ensure_stage(ctx, 5, (size_t)M * N * sizeof(float), error, error_capacity);
-    if (status != MI355Q_OK) return status;
-    void *partial = ctx->stage[5];
+    const size_t cells = (size_t)M * N;
     const uint32_t keep = flags & (MI355Q_X_DEVICE | MI355Q_ASYNC);
-    status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, residual, residual_dtype,
-                              keep | MI355Q_Y_DEVICE | (flags & (MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
-                              error, error_capacity);
+    if (weight->row_scale == nullptr) {
+        // the high part (+ the caller's residual) into fp32, then the low part on top of it
+        int status = ensure_stage(ctx, 5, cells * sizeof(float), error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        void *partial = ctx->stage[5];
+        status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, residual, residual_dtype,
+                                  keep | MI355Q_Y_DEVICE |
+                                      (flags & (MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
+                                  error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        return mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, y, y_dtype, partial, MI355Q_F32,
+                                keep | (flags & MI355Q_Y_DEVICE) | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+    }
+    // Q8 rows: the integer sum of both parts in fp32, then scale (and residual) per element
+    if (!dtype_valid(y_dtype) || (residual != nullptr && !dtype_valid(residual_dtype))) {
+        set_error(error, error_capacity, "q8_linear: y_dtype=%d residual_dtype=%d", y_dtype, residual_dtype);
+        return MI355Q_ERROR_INVALID;
+    }
+    const bool y_dev = flags & MI355Q_Y_DEVICE, r_dev = residual == nullptr || (flags & MI355Q_RESIDUAL_DEVICE);
+    const bool is_bias = flags & MI355Q_RESIDUAL_IS_BIAS;
+    if ((flags & MI355Q_ASYNC) && !(y_dev && r_dev)) {
+        set_error(error, error_capacity, "q8_linear: ASYNC needs device pointers throughout");
+        return MI355Q_ERROR_INVALID;
+    }
+    int status = ensure_stage(ctx, 5, 2u * cells * sizeof(float), error, error_capacity);
     if (status != MI355Q_OK) return status;
-    return mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, y, y_dtype, partial, MI355Q_F32,
-                            keep | (flags & MI355Q_Y_DEVICE) | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+    float *partial = (float *)ctx->stage[5], *sum = partial + cells;
+    status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, nullptr, MI355Q_F32,
+                              keep | MI355Q_Y_DEVICE, error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    status = mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, sum, MI355Q_F32, partial, MI355Q_F32,
+                              keep | MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    const size_t y_bytes = cells * dtype_bytes(y_dtype);
+    const size_t r_bytes = (is_bias ? N : cells) * dtype_bytes(residual_dtype);
+    void *y_on_device = y;
+    const void *r_on_device = residual;
+    if (!y_dev) {
+        if ((status = ensure_stage(ctx, 1, y_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        y_on_device = ctx->stage[1];
+    }
+    if (!r_dev) {
+        if ((status = ensure_stage(ctx, 2, r_bytes, error, error_capacity)) != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[2], residual, r_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "residual upload");
+        r_on_device = ctx->stage[2];
+    }
+    hipError_t launched = launch(ctx, q8rows_finish_kernel, dim3((uint32_t)((cells + 255u) / 256u)), dim3(256), 0,
+                                 (const float *)sum, (const float *)weight->row_scale, r_on_device, residual_dtype,
+                                 (int)is_bias, y_on_device, y_dtype, M, N);
+    if (launched != hipSuccess) return fail_hip(launched, "q8 rows finish launch", error, error_capacity);
+    if (!y_dev)
+        MI355Q_HIP(hipMemcpyAsync(y, y_on_device, y_bytes, hipMemcpyDeviceToHost, ctx->stream), "output download");
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q8_linear sync");
+    return MI355Q_OK;
 }

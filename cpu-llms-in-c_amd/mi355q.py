@@ -89,6 +89,7 @@ SIGNATURES = {
     "mi355q_q38_layout_field": (_int, [_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_char_p),
                                        ctypes.POINTER(_u32), ctypes.POINTER(_u32)]),
     "mi355q_q8_weight_prepare": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _int, _u32, ctypes.POINTER(ctypes.c_void_p), *_err]),
+    "mi355q_q8rows_weight_prepare": (_int, [_vp, _vp, _u32, _u32, _u32, ctypes.POINTER(ctypes.c_void_p), *_err]),
     "mi355q_q8_weight_destroy": (None, [_vp]),
     "mi355q_q8_weight_image_bytes": (ctypes.c_size_t, [_vp]),
     "mi355q_q8_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
@@ -319,6 +320,12 @@ class Context:
         out = ctypes.c_void_p()
         _call(self.lib.mi355q_q8_weight_prepare, self.handle, _ptr(quants), _ptr(meta_a), _ptr(meta_b), N, K,
               meta_kind, 0, ctypes.byref(out))
+        return out
+
+    def q8rows_prepare(self, records, N: int, K: int):
+        """Records [N][4 + K]: fp32 scale then K int8 per output row."""
+        out = ctypes.c_void_p()
+        _call(self.lib.mi355q_q8rows_weight_prepare, self.handle, _ptr(records), N, K, 0, ctypes.byref(out))
         return out
 
     def q8_destroy(self, weight):

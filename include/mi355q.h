@@ -223,6 +223,17 @@ int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void
                              const void *meta_b, uint32_t N, uint32_t K, int meta_kind,
                              uint32_t flags, mi355q_q8_weight **out,
                              char *error, size_t error_capacity);
+/* Q8 rows: per output row an fp32 scale followed by K signed bytes, w = scale * v — the
+ * MMO_Q8_ROW tensors of minimindo_thinker.c (:84-86,112-122) and the Q8 payload of
+ * minimindo_audio_encoder.c (:90,216-217), records [N][4 + K].  Prepared as two Q4 weights
+ * with integer metadata (v + 128 = 16*hi + lo), so mi355q_q8_linear on such a weight
+ * computes the exact integer-weighted sum in fp32 and multiplies it by the row's scale at
+ * the end, as q8_f32_dot's callers do (minimindo_thinker.c:124-213, q8_matvec /
+ * q8_matmul_sequence: fp32 activations in, fp32 out); a residual is added after the scale.
+ * K must be a non-zero multiple of 64. */
+int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *records, uint32_t N,
+                                 uint32_t K, uint32_t flags, mi355q_q8_weight **out,
+                                 char *error, size_t error_capacity);
 void mi355q_q8_weight_destroy(mi355q_q8_weight *weight);
 size_t mi355q_q8_weight_image_bytes(const mi355q_q8_weight *weight); /* N*K + N*(K/64)*4 */
 int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *weight, const void *x,

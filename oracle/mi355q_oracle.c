@@ -260,6 +260,31 @@ int orc_q8_affine_linear(const uint8_t *quants, const void *meta_a, const void *
     return 0;
 }
 
+/* Q8 rows x fp32 activations: records of fp32 scale + K int8 per output row (the MMO_Q8_ROW
+ * payload), out[p*N + n] = (float)(sum_k (double)x[p][k] * q[n][k]) * scale[n] -- the portable
+ * branch of q8_f32_dot and its callers q8_matvec / q8_matmul_rows
+ * (models/minimind-o/targets/generic/minimindo_thinker.c:124-213; the aarch64 branch adds
+ * in four fp32 lanes instead).  Pinned by golden vectors from that C, bit for bit. */
+void orc_q8rows_f32_linear(const uint8_t *records, uint32_t N, uint32_t K, const float *x,
+                           uint32_t M, float *out)
+{
+    const size_t stride = sizeof(float) + K;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t n = 0; n < (int64_t)N; ++n) {
+        const uint8_t *record = records + (size_t)n * stride;
+        float scale;
+        memcpy(&scale, record, sizeof scale);
+        const int8_t *values = (const int8_t *)(record + sizeof scale);
+        for (uint32_t p = 0; p < M; ++p) {
+            double sum = 0.0;
+            for (uint32_t k = 0; k < K; ++k) sum += (double)x[(size_t)p * K + k] * values[k];
+            out[(size_t)p * N + (size_t)n] = (float)sum * scale;
+        }
+    }
+}
+
 float orc_q4_dot_f16x_seq(const uint8_t *quants, const uint16_t *meta_interleaved,
                           const uint16_t *x_f16, size_t row, size_t groups)
 {

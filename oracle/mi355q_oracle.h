@@ -92,6 +92,11 @@ int orc_q8_affine_linear(const uint8_t *quants, const void *meta_a, const void *
                          const void *x, int x_kind, uint32_t M,
                          int weight_rounding, int accumulate, double *y);
 
+/* Q8 rows (fp32 scale + K int8 per row) x fp32 activations, out [M][N]:
+ * minimindo_thinker.c:124-213 (q8_f32_dot portable branch, q8_matvec, q8_matmul_rows). */
+void orc_q8rows_f32_linear(const uint8_t *records, uint32_t N, uint32_t K, const float *x,
+                           uint32_t M, float *out);
+
 /* Single-row convenience forms of the same thing. */
 float orc_q4_dot_f16x_seq(const uint8_t *quants, const uint16_t *meta_interleaved,
                           const uint16_t *x_f16, size_t row, size_t groups);

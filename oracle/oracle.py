@@ -47,6 +47,8 @@ def lib() -> ctypes.CDLL:
                                     _int, _u32, _u32, _vp, _int]
         l.orc_q8_affine_linear.restype = _int
         l.orc_q8_affine_linear.argtypes = [_vp, _vp, _vp, _int, _u32, _u32, _vp, _int, _u32, _int, _int, _vp]
+        l.orc_q8rows_f32_linear.restype = None
+        l.orc_q8rows_f32_linear.argtypes = [_vp, _u32, _u32, _vp, _u32, _vp]
         l.orc_q4_dot_f16x_seq.restype = _c.c_float
         l.orc_q4_dot_f16x_seq.argtypes = [_vp, _vp, _vp, _sz, _sz]
         l.orc_q4_dot_f32x_seq.restype = _c.c_float
@@ -104,6 +106,19 @@ def ref_minimindo():
     return _libs["minimindo"]
 
 
+def ref_thinker():
+    """The reference's compiled Q8-row x fp32 product (minimindo_thinker.c), or None if not built."""
+    if "thinker" not in _libs:
+        path = REF_MINIMINDO_PATH.with_name("libref_thinker.so")
+        if not path.exists():
+            return None
+        l = ctypes.CDLL(os.fspath(path))
+        l.ref_thinker_q8_matmul_sequence.restype = None
+        l.ref_thinker_q8_matmul_sequence.argtypes = [_vp, _u32, _u32, _vp, _u32, _vp]
+        _libs["thinker"] = l
+    return _libs["thinker"]
+
+
 # ---- convenience wrappers ---------------------------------------------------
 
 def q4_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_kind, M,
@@ -131,6 +146,14 @@ def q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, x_kind, M,
     if status != 0:
         raise ValueError(f"orc_q8_affine_linear status {status}")
     return y
+
+
+def q8rows_f32_linear(records, N, K, x):
+    """Q8 rows (fp32 scale + K int8 each) x fp32 x [M][K] -> fp32 [M][N]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty((x.shape[0], N), dtype=np.float32)
+    lib().orc_q8rows_f32_linear(_p(records), N, K, _p(x), x.shape[0], _p(out))
+    return out
 
 
 def q4_dequantize_rows(quants, meta_a, meta_b, meta_kind, K, rows):

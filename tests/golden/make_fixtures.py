@@ -72,7 +72,25 @@ def w8a8_fixture():
                         out_bias=out_bias, out_nobias=out_nobias, dots=dots)
 
 
+def q8rows_f32_fixture():
+    """The reference's q8_matvec / q8_matmul_sequence (minimindo_thinker.c:181-213) on seeded inputs."""
+    ref = oracle.ref_thinker()
+    assert ref is not None, "oracle/_ref is not built"
+    rng = np.random.default_rng(20250103)
+    N, K, M = 40, 192, 3
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    w[5] = 0.0  # all-zero row: scale 1, zero codes
+    rows = oracle.q8_weight_quantize(w)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    out = np.empty((M, N), dtype=np.float32)
+    ref.ref_thinker_q8_matmul_sequence(rows.ctypes.data, N, K, x.ctypes.data, M, out.ctypes.data)
+    out_one = np.empty((1, N), dtype=np.float32)
+    ref.ref_thinker_q8_matmul_sequence(rows.ctypes.data, N, K, x[1].ctypes.data, 1, out_one.ctypes.data)
+    np.savez_compressed(HERE / "q8rows_f32_thinker.npz", rows=rows, x=x, out=out, out_one=out_one)
+
+
 if __name__ == "__main__":
     sym128_fixture()
     w8a8_fixture()
+    q8rows_f32_fixture()
     print("wrote", sorted(p.name for p in HERE.glob("*.npz")))

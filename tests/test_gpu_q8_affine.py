@@ -68,3 +68,60 @@ def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
         print(f"distance to exact weights / rms: this library {ours:.2e}, half(scale*q+bias) {theirs:.2e}", flush=True)
         assert ours <= 2e-3 and theirs <= 2e-3
         assert float(np.max(np.abs(with_residual - (exact + residual)) / rms)) <= 2e-3
+
+
+def test_q8rows_f32_against_reference_golden(engine, oracle, gpu):
+    """Q8 rows x fp32 activations (mi355q_q8rows_weight_prepare + mi355q_q8_linear) against the
+    golden vectors of the reference's own q8_matvec / q8_matmul_sequence
+    (minimindo_thinker.c:181-213).  The reference adds in double and rounds once; here the
+    integer-weighted sum is accumulated in fp32 from activations carried as fp16 value +
+    remainder: the Q4 gate, max_i |y_i - ref_i| / max(|ref_i|, 1e-2*rms(ref)) <= 1e-3."""
+    import pathlib
+    golden = np.load(pathlib.Path(__file__).parent / "golden" / "q8rows_f32_thinker.npz", allow_pickle=False)
+    M, K = golden["x"].shape
+    N = golden["out"].shape[1]
+    weight = gpu.q8rows_prepare(golden["rows"], N, K)
+    try:
+        print("q8 rows golden case", flush=True)
+        y = gpu.q8_linear(weight, N, golden["x"], engine.F32, engine.F32)
+        one = gpu.q8_linear(weight, N, golden["x"][1:2], engine.F32, engine.F32)
+    finally:
+        gpu.q8_destroy(weight)
+    error = q4_relative_error(y, golden["out"])
+    print(f"relative error vs the reference's C: {error:.2e}", flush=True)
+    assert error <= 1e-3
+    assert q4_relative_error(one, golden["out_one"]) <= 1e-3
+    assert not y[:, 5].any()  # the all-zero row
+
+
+@pytest.mark.parametrize("N,K,M", [(768, 768, 1), (2048, 768, 6), (768, 2048, 40)])
+def test_q8rows_f32_shapes(engine, oracle, gpu, N, K, M):
+    """MiniMind-sized projections (hidden 768) at M = 1, a short sequence, and a sequence long
+    enough for the GEMM path (M > 8 rows of fp32), with a per-column bias added after the scale."""
+    rng = np.random.default_rng(N + K + M)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    rows = oracle.q8_weight_quantize(w)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    weight = gpu.q8rows_prepare(rows, N, K)
+    try:
+        print(f"q8 rows N={N} K={K} M={M}", flush=True)
+        y = gpu.q8_linear(weight, N, x, engine.F32, engine.F32)
+        _call_bias = engine.library().mi355q_q8_linear
+        biased = np.empty((M, N), dtype=np.float32)
+        message = __import__("ctypes").create_string_buffer(256)
+        status = _call_bias(gpu.handle, weight, x.ctypes.data, engine.F32, M, biased.ctypes.data, engine.F32,
+                            bias.ctypes.data, engine.F32, engine.RESIDUAL_IS_BIAS, message, 256)
+        assert status == 0, message.value
+    finally:
+        gpu.q8_destroy(weight)
+    ref = oracle.q8rows_f32_linear(rows, N, K, x).astype(np.float64)
+    if M <= 8:
+        assert q4_relative_error(y, ref) <= 1e-3
+        assert q4_relative_error(biased, ref + bias) <= 1e-3
+    else:
+        # the GEMM path rounds fp32 activations to fp16 once per call (2^-11 per element): the
+        # gate is the distance relative to the row's rms, as for the other fp16-operand paths
+        rms = np.sqrt(np.mean(ref * ref, axis=1, keepdims=True))
+        assert float(np.max(np.abs(y - ref) / rms)) <= 2e-3
+        assert float(np.max(np.abs(biased - (ref + bias)) / rms)) <= 2e-3

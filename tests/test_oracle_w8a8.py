@@ -73,3 +73,26 @@ def test_weight_quantizer_properties(oracle):
     q = rows[1, 4:].view(np.int8)
     assert q[0] == 127 and q[1] == -127 and np.all(np.abs(q.astype(int)) <= 127)
     assert np.array_equal(q, np.clip(np.rint(w[1] / scale), -127, 127).astype(np.int8))
+
+
+def test_q8rows_f32_matches_reference_golden_bitwise(oracle):
+    """orc_q8rows_f32_linear against the reference's own q8_matvec / q8_matmul_sequence
+    (minimindo_thinker.c:181-213, compiled from where it lies; golden vectors committed), bit
+    for bit, and live against oracle/_ref where that is built."""
+    golden = np.load(GOLDEN.with_name("q8rows_f32_thinker.npz"), allow_pickle=False)
+    M, K = golden["x"].shape
+    N = golden["out"].shape[1]
+    out = oracle.q8rows_f32_linear(golden["rows"], N, K, golden["x"])
+    assert np.array_equal(out.view(np.uint32), golden["out"].view(np.uint32))
+    one = oracle.q8rows_f32_linear(golden["rows"], N, K, golden["x"][1:2])
+    assert np.array_equal(one.view(np.uint32), golden["out_one"].view(np.uint32))
+    assert not out[:, 5].any()  # the all-zero row
+    ref = oracle.ref_thinker()
+    if ref is not None:
+        rng = np.random.default_rng(5)
+        w = (rng.standard_normal((24, 128)) * 0.02).astype(np.float32)
+        rows = oracle.q8_weight_quantize(w)
+        x = rng.standard_normal((5, 128)).astype(np.float32)
+        live = np.empty((5, 24), dtype=np.float32)
+        ref.ref_thinker_q8_matmul_sequence(rows.ctypes.data, 24, 128, x.ctypes.data, 5, live.ctypes.data)
+        assert np.array_equal(oracle.q8rows_f32_linear(rows, 24, 128, x).view(np.uint32), live.view(np.uint32))
