@@ -104,3 +104,13 @@ def test_forced_decompositions(engine, oracle, gpu, forced, monkeypatch):
     tile on the last wave), with and without K splits."""
     monkeypatch.setenv("MI355Q_Q4_GEMM", forced)
     run_case(engine, oracle, gpu, 1104, 2176, 150, engine.META_BF16_PLANES, engine.F16, engine.F32)
+
+
+@pytest.mark.parametrize("forced", ["6,1", "7,1", "7,2"])
+@pytest.mark.parametrize("K", [128, 256, 384, 640])
+def test_pipelined_kernel_short_rows(engine, oracle, gpu, forced, K, monkeypatch):
+    """The pipelined kernel fetches three steps ahead and rotates its registers over three
+    steps: rows of one to five 128-column steps exercise its prologue, the clamped fetches past
+    the end and both remainder steps (alone and under a K split)."""
+    monkeypatch.setenv("MI355Q_Q4_GEMM", forced)
+    run_case(engine, oracle, gpu, 560, K, 70, engine.META_BF16_PLANES, engine.F16, engine.F32)
