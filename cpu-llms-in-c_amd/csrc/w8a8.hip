@@ -82,6 +82,56 @@ quantize_i8_kernel(const float *__restrict__ x, uint32_t K, int8_t *__restrict__
     if (threadIdx.x == 0) scales[blockIdx.x] = scale;
 }
 
+// Causal convolution windows, quantized per position: window[in * kernel + k] of position t is
+// input[in][t - (kernel-1) + k], from `history` [channels][kernel-1] (or zero) before the
+// start; then the per-token quantizer above on the window.  causal_q8_positions /
+// causal_q8_windows, minimindo_mimi.c:552-598.  One workgroup per position; the window is
+// gathered twice (maximum, then codes) instead of being kept.
+// With `pairs` (transposed convolution, deconv_q8_positions, minimindo_mimi.c:631-652):
+// window[in] = input[in][t], window[channels + in] = input[in][t-1], history[in] or 0.
+__global__ void __launch_bounds__(256)
+causal_q8_windows_kernel(const float *__restrict__ input, const float *__restrict__ history,
+                         uint32_t channels, uint32_t kernel, uint32_t length, int pairs,
+                         int8_t *__restrict__ q, float *__restrict__ scales)
+{
+    __shared__ float wave_max[4];
+    const uint32_t t = blockIdx.x;
+    const uint32_t columns = pairs ? channels * 2u : channels * kernel;
+    const uint32_t before = pairs ? 1u : kernel - 1u;
+    auto element = [&](uint32_t column) {
+        uint32_t in, k;
+        if (pairs) {
+            in = column % channels;
+            k = column < channels ? 1u : 0u;  // the current sample first, then the previous one
+        } else {
+            in = column / kernel;
+            k = column % kernel;
+        }
+        const int32_t source = (int32_t)t - (int32_t)before + (int32_t)k;
+        if (source >= 0) return input[(size_t)in * length + (uint32_t)source];
+        if (history) return history[(size_t)in * before + (uint32_t)((int32_t)before + source)];
+        return 0.0f;
+    };
+    int8_t *out = q + (size_t)t * columns;
+    float maximum = 0.0f;
+    for (uint32_t c = threadIdx.x; c < columns; c += 256u) maximum = fmaxf(maximum, fabsf(element(c)));
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+    if ((threadIdx.x & 63u) == 0u) wave_max[threadIdx.x >> 6] = maximum;
+    __syncthreads();
+    maximum = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    if (!(maximum > 0.0f)) {
+        for (uint32_t c = threadIdx.x; c < columns; c += 256u) out[c] = 0;
+        if (threadIdx.x == 0) scales[t] = 0.0f;
+        return;
+    }
+    const float scale = maximum / 127.0f;
+    const float inverse = 1.0f / scale;
+    for (uint32_t c = threadIdx.x; c < columns; c += 256u)
+        out[c] = (int8_t)(int)__builtin_rintf(element(c) * inverse);
+    if (threadIdx.x == 0) scales[t] = scale;
+}
+
 struct W8a8Params {
     const uint4 *tiles;
     const float *wscales;
@@ -91,6 +141,9 @@ struct W8a8Params {
     float *out;            // [M][N]
     int32_t *acc;          // [M][N] or null
     uint32_t M, N, K, NT, KS;
+    // 0: out[m][n] = ((float)acc * wscale) * xscale + bias (matrix_i8_rows);
+    // 1: out[n][m] = bias + (wscale * xscale) * (float)acc (stream_conv_cells, minimindo_mimi.c:869-880)
+    int channel_major;
 };
 
 // A workgroup of four waves owns one tile of 16 weight rows and MB*16 activation
@@ -138,10 +191,16 @@ __global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
         if (p.acc) p.acc[at] = sum;
         {
 #pragma clang fp contract(off)
-            float value = (float)sum * p.wscales[n];
-            value = value * p.xscales[m];
-            value = value + (p.bias ? p.bias[n] : 0.0f);
-            p.out[at] = value;
+            if (p.channel_major) {
+                float value = p.wscales[n] * p.xscales[m];
+                value = value * (float)sum;
+                p.out[(size_t)n * p.M + m] = (p.bias ? p.bias[n] : 0.0f) + value;
+            } else {
+                float value = (float)sum * p.wscales[n];
+                value = value * p.xscales[m];
+                value = value + (p.bias ? p.bias[n] : 0.0f);
+                p.out[at] = value;
+            }
         }
     }
 }
@@ -259,6 +318,60 @@ int mi355q_quantize_i8(mi355q_context *ctx, const float *x, uint32_t M, uint32_t
     return MI355Q_OK;
 }
 
+int mi355q_causal_q8_windows(mi355q_context *ctx, const float *input, const float *history, uint32_t channels,
+                             uint32_t kernel, uint32_t length, int8_t *q, float *scales, uint32_t flags,
+                             char *error, size_t error_capacity)
+{
+    const bool pairs = (flags & MI355Q_WINDOWS_PAIRS) != 0;
+    if (ctx == nullptr || input == nullptr || q == nullptr || scales == nullptr || channels == 0 || length == 0 ||
+        (!pairs && kernel == 0)) {
+        set_error(error, error_capacity, "causal_q8_windows: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    const bool device = (flags & MI355Q_X_DEVICE) && (flags & MI355Q_Y_DEVICE);
+    if (!device && (flags & (MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC))) {
+        set_error(error, error_capacity, "causal_q8_windows: pointers must be all host or all device");
+        return MI355Q_ERROR_INVALID;
+    }
+    const uint32_t columns = pairs ? channels * 2u : channels * kernel;
+    const uint32_t before = pairs ? 1u : kernel - 1u;
+    const size_t in_bytes = (size_t)channels * length * sizeof(float);
+    const size_t history_bytes = (size_t)channels * before * sizeof(float);
+    const size_t q_bytes = (size_t)length * columns;
+    const float *in_dev = input, *history_dev = history;
+    int8_t *q_dev = q;
+    float *s_dev = scales;
+    if (!device) {
+        int status = ensure_stage(ctx, 0, in_bytes + history_bytes + 16u, error, error_capacity);
+        if (status == MI355Q_OK)
+            status = ensure_stage(ctx, 1, q_bytes + (size_t)length * 4u + 16u, error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        MI355Q_HIP(hipMemcpyAsync(ctx->stage[0], input, in_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "input upload");
+        in_dev = (const float *)ctx->stage[0];
+        if (history != nullptr && history_bytes != 0) {
+            char *at = (char *)ctx->stage[0] + ((in_bytes + 15u) & ~(size_t)15u);
+            MI355Q_HIP(hipMemcpyAsync(at, history, history_bytes, hipMemcpyHostToDevice, ctx->stream),
+                       "history upload");
+            history_dev = (const float *)at;
+        }
+        q_dev = (int8_t *)ctx->stage[1];
+        s_dev = (float *)((char *)ctx->stage[1] + ((q_bytes + 15u) & ~(size_t)15u));
+    }
+    if (before == 0) history_dev = nullptr;
+    hipError_t launched = launch(ctx, causal_q8_windows_kernel, dim3(length), dim3(256), 0, in_dev, history_dev,
+                                 channels, kernel, length, (int)pairs, q_dev, s_dev);
+    if (launched != hipSuccess) return fail_hip(launched, "causal windows launch", error, error_capacity);
+    if (!device) {
+        MI355Q_HIP(hipMemcpyAsync(q, q_dev, q_bytes, hipMemcpyDeviceToHost, ctx->stream), "code download");
+        MI355Q_HIP(hipMemcpyAsync(scales, s_dev, (size_t)length * 4u, hipMemcpyDeviceToHost, ctx->stream),
+                   "scale download");
+    }
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "causal_q8_windows sync");
+    return MI355Q_OK;
+}
+
 int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, const int8_t *q,
                        const float *x_scales, uint32_t M, const float *bias, float *out,
                        int32_t *acc, uint32_t flags, char *error, size_t error_capacity)
@@ -299,6 +412,7 @@ int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, co
     p.K = K;
     p.NT = weight->NT;
     p.KS = weight->KS;
+    p.channel_major = (flags & MI355Q_W8A8_CHANNEL_MAJOR) != 0;
     if (!device) {
         int status = ensure_stage(ctx, 0, q_bytes + ((s_bytes + 15u) & ~(size_t)15u) + b_bytes, error,
                                   error_capacity);

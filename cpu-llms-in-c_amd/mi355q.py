@@ -20,6 +20,7 @@ OK, ERROR_RUNTIME, ERROR_INVALID = 0, 1, 2
 F16, F32, BF16 = 0, 1, 2
 META_F16_INTERLEAVED, META_BF16_PLANES = 0, 1
 X_DEVICE, Y_DEVICE, RESIDUAL_DEVICE, ASYNC, SOURCE_DEVICE, RESIDUAL_IS_BIAS = 1, 2, 4, 8, 16, 32
+W8A8_CHANNEL_MAJOR, WINDOWS_PAIRS = 128, 256
 FUSE_GATE_UP_SILU = 64
 SYM128_ROW_MAJOR, SYM128_OUTPUT_BLOCKED = 0, 1
 
@@ -93,6 +94,7 @@ SIGNATURES = {
     "mi355q_q8_weight_destroy": (None, [_vp]),
     "mi355q_q8_weight_image_bytes": (ctypes.c_size_t, [_vp]),
     "mi355q_q8_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
+    "mi355q_causal_q8_windows": (_int, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp, _u32, *_err]),
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
@@ -441,15 +443,30 @@ class Context:
         _call(self.lib.mi355q_quantize_i8, self.handle, _ptr(x), M, K, _ptr(q), _ptr(scales), 0)
         return q, scales
 
-    def w8a8_linear(self, weight, N: int, q: np.ndarray, x_scales: np.ndarray, bias=None):
+    def w8a8_linear(self, weight, N: int, q: np.ndarray, x_scales: np.ndarray, bias=None,
+                    channel_major: bool = False):
+        """out [M][N] (or [N][M] with the streaming convolution's epilogue) and the int32 sums [M][N]."""
         q = np.ascontiguousarray(q, dtype=np.int8)
         M = q.shape[0]
-        out = np.empty((M, N), dtype=np.float32)
+        out = np.empty((N, M) if channel_major else (M, N), dtype=np.float32)
         acc = np.empty((M, N), dtype=np.int32)
         _call(self.lib.mi355q_w8a8_linear, self.handle, weight, _ptr(q),
               _ptr(np.ascontiguousarray(x_scales, dtype=np.float32)), M, _ptr(bias), _ptr(out),
-              _ptr(acc), 0)
+              _ptr(acc), W8A8_CHANNEL_MAJOR if channel_major else 0)
         return out, acc
+
+    def causal_q8_windows(self, x: np.ndarray, history, kernel: int, pairs: bool = False):
+        """x [channels][length] fp32 -> (q [length][columns] int8, scales [length])."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        channels, length = x.shape
+        columns = channels * (2 if pairs else kernel)
+        q = np.empty((length, columns), dtype=np.int8)
+        scales = np.empty(length, dtype=np.float32)
+        if history is not None:
+            history = np.ascontiguousarray(history, dtype=np.float32)
+        _call(self.lib.mi355q_causal_q8_windows, self.handle, _ptr(x), _ptr(history), channels, kernel, length,
+              _ptr(q), _ptr(scales), WINDOWS_PAIRS if pairs else 0)
+        return q, scales
 
     def quantize_i8_device(self, x_ptr: int, M: int, K: int, q_ptr: int, scales_ptr: int,
                            asynchronous: bool = True):

@@ -74,7 +74,13 @@ enum {
      * silu(g) = g / (1 + exp(-g)) in fp32; targets[1].y is not written and may be NULL; no
      * residuals.  The reference's fused decode kernel qwen38_q4_gate_up_silu
      * (qwen38_q4.metal:129-151; source_mlp_reference_first_8, qwen38_m3_pack.c:244-349) */
-    MI355Q_FUSE_GATE_UP_SILU = 1u << 6
+    MI355Q_FUSE_GATE_UP_SILU = 1u << 6,
+    /* mi355q_w8a8_linear: the streaming convolution's epilogue and layout,
+     * out[n][m] = bias[n] + (weight_scale[n] * x_scales[m]) * (float)acc
+     * (stream_conv_cells, minimindo_mimi.c:869-880) */
+    MI355Q_W8A8_CHANNEL_MAJOR = 1u << 7,
+    /* mi355q_causal_q8_windows: the two-sample windows of a transposed convolution */
+    MI355Q_WINDOWS_PAIRS = 1u << 8
 };
 
 /* record order of a symmetric group-128 Q4 tensor */
@@ -414,6 +420,22 @@ void mi355q_w8a8_weight_destroy(mi355q_w8a8_weight *weight);
 int mi355q_quantize_i8(mi355q_context *ctx, const float *x, uint32_t M, uint32_t K,
                        int8_t *q, float *scales, uint32_t flags,
                        char *error, size_t error_capacity);
+
+/* The quantized input windows of a streaming causal convolution: for every position t the
+ * window [channels][kernel] of input[in][t-(kernel-1)+k] (input is channel-major
+ * [channels][length]; samples before the start come from history [channels][kernel-1], or
+ * are zero when history is NULL), quantized per position like mi355q_quantize_i8:
+ * q [length][channels*kernel], scales [length].  Bit-exact with causal_q8_windows
+ * (minimindo_mimi.c:552-598); with MI355Q_WINDOWS_PAIRS the windows are those of
+ * deconv_q8_windows (:631-670): [input[in][t] for all in, then input[in][t-1] or
+ * history[in]], `kernel` ignored.  Followed by mi355q_w8a8_linear with
+ * MI355Q_W8A8_CHANNEL_MAJOR on the convolution's Q8 weight [out][channels*kernel] this is
+ * stream_conv1d (:882-917) without the history update, which stays with the caller.
+ * flags as for mi355q_quantize_i8. */
+int mi355q_causal_q8_windows(mi355q_context *ctx, const float *input, const float *history,
+                             uint32_t channels, uint32_t kernel, uint32_t length,
+                             int8_t *q, float *scales, uint32_t flags,
+                             char *error, size_t error_capacity);
 
 /* out[m][n] = ((float)acc[m][n] * weight_scale[n]) * x_scales[m] + bias[n], with
  * acc[m][n] = sum_k w[n][k] * q[m][k] in int32; bias may be NULL; when `acc` is

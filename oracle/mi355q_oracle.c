@@ -484,6 +484,53 @@ void orc_w8a8_linear(const uint8_t *weights, uint32_t N, uint32_t K,
     }
 }
 
+/* The streaming causal convolution of the Mimi decoder.
+ * Windows: causal_q8_positions / causal_q8_windows (minimindo_mimi.c:552-598); with `pairs`
+ * deconv_q8_positions (:631-652).  q [length][columns], scales [length]. */
+void orc_causal_q8_windows(const float *input, const float *history, uint32_t channels,
+                           uint32_t kernel, uint32_t length, int pairs, int8_t *q, float *scales)
+{
+    const uint32_t columns = pairs ? channels * 2u : channels * kernel;
+    float *window = (float *)malloc((size_t)columns * sizeof(float));
+    if (!window) return;
+    for (uint32_t t = 0; t < length; ++t) {
+        if (pairs) {
+            for (uint32_t in = 0; in < channels; ++in) {
+                window[in] = input[(size_t)in * length + t];
+                window[channels + in] = t ? input[(size_t)in * length + t - 1u] : history ? history[in] : 0.0f;
+            }
+        } else {
+            const uint32_t before = kernel - 1u;
+            for (uint32_t in = 0; in < channels; ++in)
+                for (uint32_t k = 0; k < kernel; ++k) {
+                    const int32_t source = (int32_t)t - (int32_t)before + (int32_t)k;
+                    float value = 0.0f;
+                    if (source >= 0) value = input[(size_t)in * length + (uint32_t)source];
+                    else if (history) value = history[(size_t)in * before + (uint32_t)((int32_t)before + source)];
+                    window[(size_t)in * kernel + k] = value;
+                }
+        }
+        scales[t] = orc_quantize_i8(window, q + (size_t)t * columns, columns);
+    }
+    free(window);
+}
+
+/* out[n*M + t] = bias[n] + wscale[n] * xscale[t] * dot: stream_conv_cells
+ * (minimindo_mimi.c:869-880); channel-major, product evaluated left to right. */
+void orc_w8a8_conv(const uint8_t *weights, uint32_t N, uint32_t K, const int8_t *q,
+                   const float *x_scales, uint32_t M, const float *bias, float *out)
+{
+    for (uint32_t n = 0; n < N; ++n) {
+        const uint8_t *record = weights + (size_t)n * (4u + K);
+        float weight_scale;
+        memcpy(&weight_scale, record, 4);
+        const int8_t *w = (const int8_t *)(record + 4);
+        for (uint32_t t = 0; t < M; ++t)
+            out[(size_t)n * M + t] =
+                (bias ? bias[n] : 0.0f) + weight_scale * x_scales[t] * orc_i8_dot(w, q + (size_t)t * K, K);
+    }
+}
+
 /* Per-output-row symmetric int8 weights, record = [fp32 scale][K int8].
  * Follows compiler/compile_minimindo_sensevoice_image.py:38-46 (q8_payload):
  * scale = max|w|/127 in double (1.0 for an all-zero row), stored as fp32;

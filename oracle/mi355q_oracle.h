@@ -126,6 +126,14 @@ int32_t orc_i8_dot(const int8_t *w, const int8_t *x, uint32_t count);
 void orc_w8a8_linear(const uint8_t *weights, uint32_t N, uint32_t K,
                      const int8_t *q, const float *x_scales, uint32_t M,
                      const float *bias, float *out, int32_t *acc, int threads);
+
+/* The Mimi decoder's streaming convolution: quantized causal windows
+ * (minimindo_mimi.c:552-598; pairs: :631-652) and the channel-major W8A8 product over them
+ * (:869-880).  Pinned by golden vectors of that C, bit for bit. */
+void orc_causal_q8_windows(const float *input, const float *history, uint32_t channels,
+                           uint32_t kernel, uint32_t length, int pairs, int8_t *q, float *scales);
+void orc_w8a8_conv(const uint8_t *weights, uint32_t N, uint32_t K, const int8_t *q,
+                   const float *x_scales, uint32_t M, const float *bias, float *out);
 void orc_q8_weight_quantize(const float *w, uint32_t N, uint32_t K,
                             uint8_t *rows_out);
 

@@ -49,6 +49,10 @@ def lib() -> ctypes.CDLL:
         l.orc_q8_affine_linear.argtypes = [_vp, _vp, _vp, _int, _u32, _u32, _vp, _int, _u32, _int, _int, _vp]
         l.orc_q8rows_f32_linear.restype = None
         l.orc_q8rows_f32_linear.argtypes = [_vp, _u32, _u32, _vp, _u32, _vp]
+        l.orc_causal_q8_windows.restype = None
+        l.orc_causal_q8_windows.argtypes = [_vp, _vp, _u32, _u32, _u32, _int, _vp, _vp]
+        l.orc_w8a8_conv.restype = None
+        l.orc_w8a8_conv.argtypes = [_vp, _u32, _u32, _vp, _vp, _u32, _vp, _vp]
         l.orc_q4_dot_f16x_seq.restype = _c.c_float
         l.orc_q4_dot_f16x_seq.argtypes = [_vp, _vp, _vp, _sz, _sz]
         l.orc_q4_dot_f32x_seq.restype = _c.c_float
@@ -104,6 +108,21 @@ def ref_minimindo():
                                                                  _u32, _vp, _vp]
         _libs["minimindo"] = l
     return _libs["minimindo"]
+
+
+def ref_mimi():
+    """The reference's compiled streaming convolution (minimindo_mimi.c), or None if not built."""
+    if "mimi" not in _libs:
+        path = REF_MINIMINDO_PATH.with_name("libref_mimi.so")
+        if not path.exists():
+            return None
+        l = ctypes.CDLL(os.fspath(path))
+        l.ref_mimi_causal_q8_windows.restype = _int
+        l.ref_mimi_causal_q8_windows.argtypes = [_vp, _vp, _u32, _u32, _u32, _vp, _vp]
+        l.ref_mimi_stream_conv1d.restype = _int
+        l.ref_mimi_stream_conv1d.argtypes = [_vp, _vp, _u32, _u32, _u32, _vp, _vp, _u32, _vp]
+        _libs["mimi"] = l
+    return _libs["mimi"]
 
 
 def ref_thinker():
@@ -202,6 +221,28 @@ def w8a8_linear(weights, N, K, q, x_scales, bias=None, threads=0):
                           _p(np.ascontiguousarray(x_scales, dtype=np.float32)), M, _p(bias),
                           _p(out), _p(acc), threads)
     return out, acc
+
+
+def causal_q8_windows(x, history, kernel, pairs=False):
+    """x [channels][length] fp32 -> (q [length][columns] int8, scales [length])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    channels, length = x.shape
+    columns = channels * (2 if pairs else kernel)
+    q = np.empty((length, columns), dtype=np.int8)
+    scales = np.empty(length, dtype=np.float32)
+    if history is not None:
+        history = np.ascontiguousarray(history, dtype=np.float32)
+    lib().orc_causal_q8_windows(_p(x), _p(history), channels, kernel, length, int(pairs), _p(q), _p(scales))
+    return q, scales
+
+
+def w8a8_conv(weights, N, K, q, x_scales, bias=None):
+    """Channel-major [N][M] output of the streaming convolution's W8A8 product."""
+    M = q.shape[0]
+    out = np.empty((N, M), dtype=np.float32)
+    lib().orc_w8a8_conv(_p(weights), N, K, _p(np.ascontiguousarray(q)),
+                        _p(np.ascontiguousarray(x_scales, dtype=np.float32)), M, _p(bias), _p(out))
+    return out
 
 
 def q8_weight_quantize(w):

@@ -89,8 +89,46 @@ def q8rows_f32_fixture():
     np.savez_compressed(HERE / "q8rows_f32_thinker.npz", rows=rows, x=x, out=out, out_one=out_one)
 
 
+def mimi_conv_fixture():
+    """The reference's causal_q8_windows and stream_conv1d (minimindo_mimi.c:552-598,869-917): two
+    consecutive chunks of a stream (the second starts from the history the first left), kernel 7
+    and kernel 1, and a chunk shorter than the history."""
+    ref = oracle.ref_mimi()
+    assert ref is not None, "oracle/_ref is not built"
+    rng = np.random.default_rng(20250104)
+    out = {}
+    for tag, (C, O, kernel, lengths) in {"k7": (16, 24, 7, (9, 4, 12)), "k1": (32, 8, 1, (5,))}.items():
+        w = (rng.standard_normal((O, C * kernel)) * 0.05).astype(np.float32)
+        rows = oracle.q8_weight_quantize(w)
+        bias = rng.standard_normal(O).astype(np.float32)
+        history = np.zeros((C, max(kernel - 1, 1)), dtype=np.float32)[:, :kernel - 1].copy()
+        out[f"{tag}_rows"], out[f"{tag}_bias"] = rows, bias
+        out[f"{tag}_shape"] = np.array([C, O, kernel], dtype=np.int64)
+        for index, length in enumerate(lengths):
+            x = rng.standard_normal((C, length)).astype(np.float32)
+            if index == 1:
+                x[:, 1] = 0.0
+            before = history.copy()
+            q = np.empty((length, C * kernel), dtype=np.int8)
+            scales = np.empty(length, dtype=np.float32)
+            history_arg = before.ctypes.data if kernel > 1 else None
+            assert ref.ref_mimi_causal_q8_windows(x.ctypes.data, history_arg, C, kernel, length, q.ctypes.data,
+                                                  scales.ctypes.data) == 0
+            y = np.empty((O, length), dtype=np.float32)
+            state = history.copy() if kernel > 1 else np.zeros(1, dtype=np.float32)
+            assert ref.ref_mimi_stream_conv1d(rows.ctypes.data, bias.ctypes.data, C, O, kernel, state.ctypes.data,
+                                              x.ctypes.data, length, y.ctypes.data) == 0
+            if kernel > 1:
+                history = state
+            for name, value in (("x", x), ("history_before", before), ("q", q), ("scales", scales), ("y", y),
+                                ("history_after", history.copy())):
+                out[f"{tag}_{index}_{name}"] = value
+    np.savez_compressed(HERE / "mimi_stream_conv.npz", **out)
+
+
 if __name__ == "__main__":
     sym128_fixture()
     w8a8_fixture()
     q8rows_f32_fixture()
+    mimi_conv_fixture()
     print("wrote", sorted(p.name for p in HERE.glob("*.npz")))

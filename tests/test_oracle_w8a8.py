@@ -96,3 +96,29 @@ def test_q8rows_f32_matches_reference_golden_bitwise(oracle):
         live = np.empty((5, 24), dtype=np.float32)
         ref.ref_thinker_q8_matmul_sequence(rows.ctypes.data, 24, 128, x.ctypes.data, 5, live.ctypes.data)
         assert np.array_equal(oracle.q8rows_f32_linear(rows, 24, 128, x).view(np.uint32), live.view(np.uint32))
+
+
+def test_mimi_stream_conv_matches_reference_golden_bitwise(oracle):
+    """orc_causal_q8_windows + orc_w8a8_conv against the reference's own causal_q8_windows and
+    stream_conv1d (minimindo_mimi.c:552-598,869-917; golden vectors of consecutive stream
+    chunks, committed), bit for bit; the pair windows of the transposed convolution against a
+    direct numpy construction."""
+    golden = np.load(GOLDEN.with_name("mimi_stream_conv.npz"), allow_pickle=False)
+    for tag, chunks in (("k7", 3), ("k1", 1)):
+        C, O, kernel = (int(v) for v in golden[f"{tag}_shape"])
+        for index in range(chunks):
+            x = golden[f"{tag}_{index}_x"]
+            history = golden[f"{tag}_{index}_history_before"] if kernel > 1 else None
+            q, scales = oracle.causal_q8_windows(x, history, kernel)
+            assert np.array_equal(q, golden[f"{tag}_{index}_q"])
+            assert np.array_equal(scales.view(np.uint32), golden[f"{tag}_{index}_scales"].view(np.uint32))
+            y = oracle.w8a8_conv(golden[f"{tag}_rows"], O, C * kernel, q, scales, golden[f"{tag}_bias"])
+            assert np.array_equal(y.view(np.uint32), golden[f"{tag}_{index}_y"].view(np.uint32))
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((6, 5)).astype(np.float32)
+    history = rng.standard_normal(6).astype(np.float32)
+    q, scales = oracle.causal_q8_windows(x, history, 0, pairs=True)
+    previous = np.concatenate([history[:, None], x[:, :-1]], axis=1)
+    windows = np.concatenate([x.T, previous.T], axis=1)
+    expect_q, expect_scales = oracle.quantize_i8(windows)
+    assert np.array_equal(q, expect_q) and np.array_equal(scales, expect_scales)
