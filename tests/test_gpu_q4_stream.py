@@ -287,6 +287,33 @@ def test_row_subsets(engine, oracle, gpu, M, x_dtype, meta_kind):
     assert q4_relative_error(gathered, full[:, ids].astype(np.float64)) <= 1e-4
 
 
+def test_row_subset_with_device_ids(engine, oracle, gpu):
+    """Row ids that already live on the GPU (MI355Q_SOURCE_DEVICE, asynchronous call): an id past
+    the matrix yields 0 instead of being refused, the rest equals the host-id call bit for bit."""
+    N, K, M = 777, 1024, 2
+    quants, meta_a, meta_b = engine.synth_q4_affine(61, 0.02, N, K, engine.META_BF16_PLANES)
+    x = make_x(engine, 62, M, K, engine.F16)
+    ids = np.array([5, N - 1, N + 3, 0, 400, 2**31, 17], dtype=np.uint32)
+    good = ids < N
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+    pointers = []
+    try:
+        print("row subset, device ids", flush=True)
+        host = gpu.q4_linear_rows(weight, ids[good], x, engine.F16, engine.F32)
+        ids_ptr, x_ptr = gpu.to_device(ids), gpu.to_device(x)
+        y_ptr = gpu.alloc(M * ids.size * 4)
+        pointers += [ids_ptr, x_ptr, y_ptr]
+        gpu.q4_linear_rows_device(weight, ids_ptr, ids.size, x_ptr, engine.F16, M, y_ptr, engine.F32)
+        gpu.sync()
+        y = gpu.download(y_ptr, (M, ids.size), np.float32)
+    finally:
+        for pointer in pointers:
+            gpu.free(pointer)
+        weight.destroy()
+    assert not y[:, ~good].any()
+    assert np.array_equal(y[:, good].view(np.uint32), host.view(np.uint32))
+
+
 def test_slices_added_in_kernel_match_second_kernel(engine, oracle, gpu, monkeypatch):
     """K slices are added by the last workgroup of a column to arrive, which needs the
     workgroups of a column on one XCD (probed when a context is created).  The probe must
