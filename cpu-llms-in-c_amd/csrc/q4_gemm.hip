@@ -739,7 +739,7 @@ q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__re
 
 // The pipelined kernel's stage is larger than the 64 KiB a kernel gets without asking: the
 // limit is raised once per device and instantiation.
-template <bool XT>
+template <int NTW, bool XT>
 static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &p)
 {
     static bool raised[64] = {};
@@ -747,12 +747,12 @@ static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &
     const int device = ctx->device;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
     if (!raised[device]) {
-        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, 4, XT>,
+        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, NTW, XT>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (status != hipSuccess) return status;
         raised[device] = true;
     }
-    return launch(ctx, q4_gemm_pipe_kernel<128, 4, XT>, grid, dim3(256), bytes, p);
+    return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT>, grid, dim3(256), bytes, p);
 }
 
 int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
@@ -803,7 +803,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     static const Variant variants[] = {
         {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
         {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
-        {128, 4, 0, 1, 0.685, 0.685, 13.0}, {128, 4, 1, 1, 0.654, 0.654, 16.5}};
+        {128, 4, 0, 1, 0.685, 0.685, 13.0}, {128, 4, 1, 1, 0.654, 0.654, 16.5},
+        {128, 5, 0, 1, 0.580, 0.580, 13.0}};
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     int best = 0;
     uint32_t best_splits = 1;
@@ -887,8 +888,9 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     case 3: launched = launch(ctx, q4_gemm_kernel<64, 4, true>, grid, dim3(256), 0, p); break;
     case 4: launched = launch(ctx, q4_gemm_kernel<64, 2, false>, grid, dim3(256), 0, p); break;
     case 5: launched = launch(ctx, q4_gemm_kernel<64, 2, true>, grid, dim3(256), 0, p); break;
-    case 6: launched = launch_pipe<false>(ctx, grid, p); break;
-    default: launched = launch_pipe<true>(ctx, grid, p); break;
+    case 6: launched = launch_pipe<4, false>(ctx, grid, p); break;
+    case 7: launched = launch_pipe<4, true>(ctx, grid, p); break;
+    default: launched = launch_pipe<5, false>(ctx, grid, p); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);

@@ -98,7 +98,7 @@ def test_dtypes_and_residual(engine, oracle, gpu, x_dtype, y_dtype):
              getattr(engine, y_dtype), residual=True)
 
 
-@pytest.mark.parametrize("forced", ["0,1", "1,2", "2,1", "3,1", "3,3", "4,1", "5,2", "6,1", "6,3", "7,1", "7,2"])
+@pytest.mark.parametrize("forced", ["0,1", "1,2", "2,1", "3,1", "3,3", "4,1", "5,2", "6,1", "6,3", "7,1", "7,2", "8,1", "8,2"])
 def test_forced_decompositions(engine, oracle, gpu, forced, monkeypatch):
     """Every kernel variant the host heuristic can pick (rows per block, tiles per wave, odd
     tile on the last wave), with and without K splits."""
@@ -106,7 +106,7 @@ def test_forced_decompositions(engine, oracle, gpu, forced, monkeypatch):
     run_case(engine, oracle, gpu, 1104, 2176, 150, engine.META_BF16_PLANES, engine.F16, engine.F32)
 
 
-@pytest.mark.parametrize("forced", ["6,1", "7,1", "7,2"])
+@pytest.mark.parametrize("forced", ["6,1", "7,1", "7,2", "8,1"])
 @pytest.mark.parametrize("K", [128, 256, 384, 640])
 def test_pipelined_kernel_short_rows(engine, oracle, gpu, forced, K, monkeypatch):
     """The pipelined kernel fetches three steps ahead and rotates its registers over three
