@@ -46,6 +46,7 @@ struct GemmParams {
     uint32_t splits, steps_per_split;
     int y_dtype, residual_dtype;
     int residual_is_bias;  // residual is one row [N], added to every activation row
+    int wide_stores;       // N % 4 == 0 and y 16-byte aligned: four adjacent outputs go out as one store
 };
 
 __device__ __forceinline__ half8 dequant8(uint32_t word, const NibbleMasks &masks, half8 scale,
@@ -102,6 +103,60 @@ __device__ __forceinline__ void store_fragment(const GemmParams &p, uint32_t spl
                 value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? n : at);
             store_from_float(p.y, p.y_dtype, at, value);
         }
+    }
+}
+
+__device__ __forceinline__ uint32_t bf16_bits(float v)  // round to nearest even
+{
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+}
+
+// The pipelined kernel multiplies with the weight tile as the first operand, which transposes the
+// result: lane (r, kq) holds row `m` = 16*i + r and the four adjacent columns n0 .. n0 + 3,
+// n0 = 16*tile + 4*kq.  They leave as one 8- or 16-byte store (a quarter of the store
+// instructions of the column-per-lane layout, whose 2-byte stores took 5 us per workgroup).
+template <int MODE>
+__device__ __forceinline__ void store_columns(const GemmParams &p, uint32_t split, uint32_t m, uint32_t n0,
+                                              const floatx4 &values)
+{
+    if (m >= p.M || n0 >= p.N) return;
+    const size_t at = (size_t)m * p.N + n0;
+    if (p.wide_stores) {  // then n0 + 3 < N as well
+        if (MODE == 0) {
+            typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+            const half4v packed = {(_Float16)values[0], (_Float16)values[1], (_Float16)values[2],
+                                   (_Float16)values[3]};
+            *(half4v *)((_Float16 *)p.y + at) = packed;
+            return;
+        }
+        if (MODE == 1) {
+            *(floatx4 *)((float *)p.y + at) = values;
+            return;
+        }
+        if (MODE == 2) {
+            const uint32_t b0 = bf16_bits(values[0]), b1 = bf16_bits(values[1]);
+            const uint32_t b2 = bf16_bits(values[2]), b3 = bf16_bits(values[3]);
+            *(uint2 *)((uint16_t *)p.y + at) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+            return;
+        }
+        if (p.splits > 1u) {
+            *(floatx4 *)(p.partials + (size_t)split * p.M * p.N + at) = values;
+            return;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t n = n0 + j;
+        if (n >= p.N) break;
+        if (p.splits > 1u) {
+            p.partials[(size_t)split * p.M * p.N + at + j] = values[j];
+            continue;
+        }
+        float value = values[j];
+        if (p.residual)
+            value += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? n : at + j);
+        store_from_float(p.y, p.y_dtype, at + j, value);
     }
 }
 
@@ -547,7 +602,8 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     auto touch_shared = [&]() { touch(a_shared[0], a_shared[1]); };
     auto multiply = [&](floatx4 &c, const half8 &a, const half2v (&b)[4]) {
         const half8 b8 = {b[0].x, b[0].y, b[1].x, b[1].y, b[2].x, b[2].y, b[3].x, b[3].y};
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b8));
+        // weights first: the result comes out transposed (see store_columns)
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %2, %1, %0" : "+a"(c) : "v"(a), "v"(b8));
     };
     // Dequantization of one quarter = NTX tiles x 4 pieces (two of a lane's eight weights each),
     // each piece three dependent vector instructions: mask-and-merge into an fp16 with the code in
@@ -684,24 +740,23 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     for (int set = 0; set < 3; ++set) landed(b_codes[set], b_meta[set]);
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- lane (r, kq) holds rows 16*i + 4*kq + j of column tile*16 + r
+    // ---- lane (r, kq) holds row 16*i + r, columns tile*16 + 4*kq .. + 3
     auto store_all = [&](auto mode) {
 #pragma unroll
         for (int t = 0; t < NTW; ++t) {
             const uint32_t tile = tile0 + t;
-            const uint32_t n = tile * kTileRows + r;
-            if (tile >= p.NT || n >= p.N) continue;
+            if (tile >= p.NT) continue;
 #pragma unroll
             for (int i = 0; i < MI; ++i)
-                store_fragment<decltype(mode)::value>(p, split, m0 + 16u * i, kq, n, acc[i][t]);
+                store_columns<decltype(mode)::value>(p, split, m0 + 16u * i + r, tile * kTileRows + 4u * kq,
+                                                     acc[i][t]);
         }
         if (XT) {
-            const uint32_t n = shared_tile * kTileRows + r;
-            if (shared_tile < p.NT && n < p.N) {
+            if (shared_tile < p.NT) {
 #pragma unroll
                 for (int i = 0; i < XI; ++i)
-                    store_fragment<decltype(mode)::value>(p, split, m0 + 16u * (XI * wave + i), kq, n,
-                                                          acc_shared[i]);
+                    store_columns<decltype(mode)::value>(p, split, m0 + 16u * (XI * wave + i) + r,
+                                                         shared_tile * kTileRows + 4u * kq, acc_shared[i]);
             }
         }
     };
@@ -785,26 +840,36 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     p.y_dtype = a.y_dtype;
     p.residual_dtype = a.residual_dtype;
     p.residual_is_bias = a.residual_is_bias;
+    p.wide_stores = w.N % 4u == 0u && (uintptr_t)p.y % 16u == 0u;
 
     // Decomposition: BM rows x (4*NTW + EXTRA) tiles per workgroup, K split in `splits`.
     // The choice minimises a microsecond estimate fitted to sweeps over every variant
     // and split on this GPU.  Kernels 0-5: a workgroup that has a compute unit to itself
     // sustains `alone` of the matrix-instruction peak, co-resident workgroups `shared`
     // together; a grid that is not a whole number of resident sets pays ~0.3 of a workgroup
-    // time for its ragged end.  The pipelined kernel (6, 7; one workgroup per compute unit)
-    // runs in whole rounds of `alone` of the peak plus `round_us` each.  A K split pays for
-    // its fp32 partials at ~4 TB/s.
+    // time for its ragged end.  The pipelined kernel (6, 7, 8; one workgroup per compute unit)
+    // runs in rounds of `step_us` per 128-column step; a round that does not fill the chip is
+    // shorter (partial_round).  A K split pays for writing its fp32
+    // partials and for the kernel that adds them.
     struct Variant {
         int bm, ntw, extra;
         int resident;          // workgroups that fit one compute unit (registers, LDS)
         double alone, shared;  // fraction of matrix-instruction peak, one / several per CU
-        double round_us;       // pipelined kernel: fixed time per round of workgroups
+        double step_us;        // pipelined kernel: measured time of one 128-column step, chip full
     };
     static const Variant variants[] = {
         {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
         {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
-        {128, 4, 0, 1, 0.685, 0.685, 13.0}, {128, 4, 1, 1, 0.654, 0.654, 16.5},
-        {128, 5, 0, 1, 0.580, 0.580, 13.0}};
+        {128, 4, 0, 1, 0.0, 0.0, 1.493}, {128, 4, 1, 1, 0.0, 0.0, 1.675}, {128, 5, 0, 1, 0.0, 0.0, 1.849}};
+    // A round of the pipelined kernel that fills only the fraction r of the compute units runs
+    // faster than a full one: the chip is power limited, and up to about half of it the clock
+    // stays near its maximum, from there it falls to the sustained clock of a full chip
+    // (fitted, like the other figures here, to interleaved timings of every variant and split
+    // at M = 256 .. 4096 on the 27B shapes: 4 % rms, the fastest choice found in 13 of 14 cases).
+    auto partial_round = [](double r) {
+        const double over = (1.0 - r) / 0.438;
+        return r <= 0.562 ? 0.771 - 0.081 * r / 0.562 : 1.0 - 0.31 * over * over;
+    };
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     int best = 0;
     uint32_t best_splits = 1;
@@ -829,11 +894,12 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             const double peak_us = (double)steps * tiles_per_wave * (c.bm / 16.0) * 64.0 / 2400.0;
             double cost;
             if (v >= 6) {
-                // a last round that leaves compute units idle runs at a higher clock (power)
-                const double round = peak_us / c.alone;
+                // 7.6 us per launch; a round = 7.2 us (fill, and the burst of stores at its end)
+                // plus its steps
                 const uint64_t rest = groups % cus;
-                cost = (double)(groups / cus) * (round + c.round_us) +
-                       (rest ? round * (0.8 + 0.2 * rest / cus) + c.round_us : 0.0);
+                const double round = 7.2 + (double)steps * c.step_us;
+                cost = 7.6 + round * ((double)(groups / cus) + (rest ? partial_round((double)rest / cus) : 0.0));
+                if (splits > 1 && c.ntw == 5) cost += 0.07 * steps * c.step_us;  // 20 tiles of fp32 to write
             }
             else if (groups <= cus)
                 cost = peak_us / c.alone;
@@ -845,8 +911,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             }
             else
                 cost = ((double)groups / slots + (groups % slots ? 0.31 : 0.0)) * c.resident * peak_us / c.shared;
-            if (splits > 1)  // fp32 partials written and read back
-                cost += 2.0 * splits * a.M * (double)w.N * 4.0 / 4.0e12 * 1.0e6;
+            if (splits > 1)  // fp32 partials at 4.6 TB/s and the kernel that adds them
+                cost += (double)splits * a.M * (double)w.N * 4.0 / 4.63e6 + 6.3;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;
