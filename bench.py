@@ -284,8 +284,7 @@ def bench_w8a8(engine, ctx, args):
     def run_steps(steps):
         for _ in range(steps):
             ctx.quantize_i8_device(x_ptr, M, K, q_ptr, s_ptr)
-            for i in range(count):
-                ctx.w8a8_linear_device(weights[i], q_ptr, s_ptr, M, bias_ptr[i], out_ptr[i], acc_ptr[i])
+            ctx.w8a8_linear_multi_device(weights, q_ptr, s_ptr, M, bias_ptr, out_ptr, acc_ptr)
 
     wall, gpu_ms, kernel_ms, launches = time_steps(ctx, run_steps, args.steps, args.warmup)
     step_ops = 2.0 * M * K * N * count
@@ -302,7 +301,8 @@ def bench_w8a8(engine, ctx, args):
         "config": {
             "workload": "per-token int8 quantization then %d projections M=%d K=%d N=%d with bias"
                         % (count, M, K, N),
-            "launches_per_step": 1 + count,
+            "launches_per_step": 2,
+            "projections_share_one_launch": True,
             "algorithmic_ops_per_step": step_ops,
             "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
             **device_fields(ctx.info()),

@@ -132,15 +132,20 @@ causal_q8_windows_kernel(const float *__restrict__ input, const float *__restric
     if (threadIdx.x == 0) scales[t] = scale;
 }
 
+constexpr uint32_t kW8a8Targets = 4;
+// Up to four weights of the same K against one quantized activation: workgroup ranges map to
+// weights (first_tile), one launch.
 struct W8a8Params {
-    const uint4 *tiles;
-    const float *wscales;
+    const uint4 *tiles[kW8a8Targets];
+    const float *wscales[kW8a8Targets];
+    const float *bias[kW8a8Targets];  // [N] or null
+    float *out[kW8a8Targets];         // [M][N]
+    int32_t *acc[kW8a8Targets];       // [M][N] or null
+    uint32_t N[kW8a8Targets], first_tile[kW8a8Targets];
+    uint32_t targets;
     const int8_t *q;       // [M][K]
     const float *xscales;  // [M]
-    const float *bias;     // [N] or null
-    float *out;            // [M][N]
-    int32_t *acc;          // [M][N] or null
-    uint32_t M, N, K, NT, KS;
+    uint32_t M, K, KS;
     // 0: out[m][n] = ((float)acc * wscale) * xscale + bias (matrix_i8_rows);
     // 1: out[n][m] = bias + (wscale * xscale) * (float)acc (stream_conv_cells, minimindo_mimi.c:869-880)
     int channel_major;
@@ -148,32 +153,55 @@ struct W8a8Params {
 
 // A workgroup of four waves owns one tile of 16 weight rows and MB*16 activation
 // rows; the waves split the 64-column steps (wave w: steps w, w+4, ...) and add
-// their int32 partial sums through LDS.
+// their int32 partial sums through LDS.  A wave fetches four of its steps (weights and
+// activations) before the first matrix instruction: at K = 1024 that is all of them, one
+// round trip to memory instead of four.
 template <int MB>
 __global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
 {
     __shared__ int red[4][MB][4][64];
+    constexpr int AHEAD = 4;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15u, kq = lane >> 4;
-    const uint32_t tile = blockIdx.x;
+    uint32_t target = 0;
+#pragma unroll
+    for (uint32_t t = 1; t < kW8a8Targets; ++t)
+        if (t < p.targets && blockIdx.x >= p.first_tile[t]) target = t;
+    const uint32_t tile = blockIdx.x - p.first_tile[target];
     const uint32_t m0 = blockIdx.y * (MB * 16u);
+    const uint32_t N = p.N[target];
 
     intx4 acc[MB];
 #pragma unroll
     for (int i = 0; i < MB; ++i) acc[i] = intx4{0, 0, 0, 0};
-    const uint4 *tile_words = p.tiles + (size_t)tile * p.KS * 64u + lane;
-    for (uint32_t ks = wave; ks < p.KS; ks += 4u) {
-        const intx4 b = __builtin_bit_cast(intx4, tile_words[(size_t)ks * 64u]);
-        const uint32_t k = ks * 64u + kq * 16u;
+    const uint4 *tile_words = p.tiles[target] + (size_t)tile * p.KS * 64u + lane;
+    const int8_t *q_rows[MB];
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-            const uint32_t m = m0 + 16u * i + r;
-            uint4 a = make_uint4(0u, 0u, 0u, 0u);
-            if (m < p.M && k < p.K) a = *(const uint4 *)(p.q + (size_t)m * p.K + k);
-            acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), b, acc[i],
-                                                           0, 0, 0);
+    for (int i = 0; i < MB; ++i) {
+        const uint32_t m = m0 + 16u * i + r;
+        q_rows[i] = m < p.M ? p.q + (size_t)m * p.K : nullptr;
+    }
+    for (uint32_t first = wave; first < p.KS; first += 4u * AHEAD) {
+        uint4 b[AHEAD], a[AHEAD][MB];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const uint32_t ks = first + 4u * u;
+            const uint32_t k = ks * 64u + kq * 16u;
+            b[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (ks < p.KS) b[u] = tile_words[(size_t)ks * 64u];
+#pragma unroll
+            for (int i = 0; i < MB; ++i) {
+                a[u][i] = make_uint4(0u, 0u, 0u, 0u);
+                if (ks < p.KS && q_rows[i] != nullptr && k < p.K) a[u][i] = *(const uint4 *)(q_rows[i] + k);
+            }
         }
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+                acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a[u][i]),
+                                                               __builtin_bit_cast(intx4, b[u]), acc[i], 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < MB; ++i)
@@ -181,25 +209,28 @@ __global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
         for (int j = 0; j < 4; ++j) red[wave][i][j][lane] = acc[i][j];
     __syncthreads();
     // lane (r, kq) of fragment i holds activation rows 16*i + 4*kq + j, weight row 16*tile + r
+    const float *wscales = p.wscales[target], *bias = p.bias[target];
+    float *out = p.out[target];
+    int32_t *acc_out = p.acc[target];
     for (uint32_t e = threadIdx.x; e < MB * 4u * 64u; e += 256u) {
         const uint32_t l = e & 63u, j = (e >> 6) & 3u, i = e >> 8;
         const int sum = red[0][i][j][l] + red[1][i][j][l] + red[2][i][j][l] + red[3][i][j][l];
         const uint32_t m = m0 + 16u * i + 4u * (l >> 4) + j;
         const uint32_t n = tile * 16u + (l & 15u);
-        if (m >= p.M || n >= p.N) continue;
-        const size_t at = (size_t)m * p.N + n;
-        if (p.acc) p.acc[at] = sum;
+        if (m >= p.M || n >= N) continue;
+        const size_t at = (size_t)m * N + n;
+        if (acc_out) acc_out[at] = sum;
         {
 #pragma clang fp contract(off)
             if (p.channel_major) {
-                float value = p.wscales[n] * p.xscales[m];
+                float value = wscales[n] * p.xscales[m];
                 value = value * (float)sum;
-                p.out[(size_t)n * p.M + m] = (p.bias ? p.bias[n] : 0.0f) + value;
+                out[(size_t)n * p.M + m] = (bias ? bias[n] : 0.0f) + value;
             } else {
-                float value = (float)sum * p.wscales[n];
+                float value = (float)sum * wscales[n];
                 value = value * p.xscales[m];
-                value = value + (p.bias ? p.bias[n] : 0.0f);
-                p.out[at] = value;
+                value = value + (bias ? bias[n] : 0.0f);
+                out[at] = value;
             }
         }
     }
@@ -372,18 +403,29 @@ int mi355q_causal_q8_windows(mi355q_context *ctx, const float *input, const floa
     return MI355Q_OK;
 }
 
-int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, const int8_t *q,
-                       const float *x_scales, uint32_t M, const float *bias, float *out,
-                       int32_t *acc, uint32_t flags, char *error, size_t error_capacity)
+int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targets, uint32_t count,
+                             const int8_t *q, const float *x_scales, uint32_t M, uint32_t flags,
+                             char *error, size_t error_capacity)
 {
-    if (ctx == nullptr || weight == nullptr || q == nullptr || x_scales == nullptr || out == nullptr ||
-        M == 0) {
-        set_error(error, error_capacity, "w8a8_linear: invalid argument");
+    if (ctx == nullptr || targets == nullptr || count == 0 || count > kW8a8Targets || q == nullptr ||
+        x_scales == nullptr || M == 0) {
+        set_error(error, error_capacity, "w8a8_linear: invalid argument (1 to %u targets)", kW8a8Targets);
         return MI355Q_ERROR_INVALID;
     }
-    if (weight->ctx != ctx) {
-        set_error(error, error_capacity, "w8a8_linear: weight belongs to another context");
-        return MI355Q_ERROR_INVALID;
+    for (uint32_t t = 0; t < count; ++t) {
+        if (targets[t].weight == nullptr || targets[t].out == nullptr) {
+            set_error(error, error_capacity, "w8a8_linear: target %u has no weight or no output", t);
+            return MI355Q_ERROR_INVALID;
+        }
+        if (targets[t].weight->ctx != ctx) {
+            set_error(error, error_capacity, "w8a8_linear: weight belongs to another context");
+            return MI355Q_ERROR_INVALID;
+        }
+        if (targets[t].weight->K != targets[0].weight->K) {
+            set_error(error, error_capacity, "w8a8_linear: targets share the activation, so their K must agree (%u, %u)",
+                      targets[0].weight->K, targets[t].weight->K);
+            return MI355Q_ERROR_INVALID;
+        }
     }
     const bool device = (flags & MI355Q_X_DEVICE) && (flags & MI355Q_Y_DEVICE);
     if (!device && (flags & (MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC))) {
@@ -395,62 +437,94 @@ int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, co
         return MI355Q_ERROR_INVALID;
     }
     MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
-    const uint32_t N = weight->N, K = weight->K;
-    const size_t q_bytes = ((size_t)M * K + 15u) & ~(size_t)15u, s_bytes = (size_t)M * 4u;
-    const size_t b_bytes = (size_t)N * 4u, o_bytes = (size_t)M * N * 4u;
+    const uint32_t K = targets[0].weight->K;
+    const size_t q_bytes = ((size_t)M * K + 15u) & ~(size_t)15u, s_bytes = ((size_t)M * 4u + 15u) & ~(size_t)15u;
     W8a8Params p;
     memset(&p, 0, sizeof p);
-    p.tiles = weight->tiles;
-    p.wscales = weight->scales;
     p.q = q;
     p.xscales = x_scales;
-    p.bias = bias;
-    p.out = out;
-    p.acc = acc;
     p.M = M;
-    p.N = N;
     p.K = K;
-    p.NT = weight->NT;
-    p.KS = weight->KS;
+    p.KS = targets[0].weight->KS;
+    p.targets = count;
     p.channel_major = (flags & MI355Q_W8A8_CHANNEL_MAJOR) != 0;
+    uint32_t tiles = 0;
+    size_t bias_bytes = 0, out_bytes = 0;
+    for (uint32_t t = 0; t < count; ++t) {
+        const mi355q_w8a8_weight *weight = targets[t].weight;
+        p.tiles[t] = weight->tiles;
+        p.wscales[t] = weight->scales;
+        p.bias[t] = targets[t].bias;
+        p.out[t] = targets[t].out;
+        p.acc[t] = targets[t].acc;
+        p.N[t] = weight->N;
+        p.first_tile[t] = tiles;
+        tiles += weight->NT;
+        bias_bytes += (size_t)weight->N * 4u;
+        out_bytes += (size_t)M * weight->N * 4u * (targets[t].acc ? 2u : 1u);
+    }
     if (!device) {
-        int status = ensure_stage(ctx, 0, q_bytes + ((s_bytes + 15u) & ~(size_t)15u) + b_bytes, error,
-                                  error_capacity);
-        if (status == MI355Q_OK) status = ensure_stage(ctx, 1, 2u * o_bytes, error, error_capacity);
+        int status = ensure_stage(ctx, 0, q_bytes + s_bytes + bias_bytes, error, error_capacity);
+        if (status == MI355Q_OK) status = ensure_stage(ctx, 1, out_bytes, error, error_capacity);
         if (status != MI355Q_OK) return status;
         char *in = (char *)ctx->stage[0];
         MI355Q_HIP(hipMemcpyAsync(in, q, (size_t)M * K, hipMemcpyHostToDevice, ctx->stream), "code upload");
         p.q = (const int8_t *)in;
         in += q_bytes;
-        MI355Q_HIP(hipMemcpyAsync(in, x_scales, s_bytes, hipMemcpyHostToDevice, ctx->stream),
+        MI355Q_HIP(hipMemcpyAsync(in, x_scales, (size_t)M * 4u, hipMemcpyHostToDevice, ctx->stream),
                    "scale upload");
         p.xscales = (const float *)in;
-        in += (s_bytes + 15u) & ~(size_t)15u;
-        if (bias) {
-            MI355Q_HIP(hipMemcpyAsync(in, bias, b_bytes, hipMemcpyHostToDevice, ctx->stream),
-                       "bias upload");
-            p.bias = (const float *)in;
+        in += s_bytes;
+        char *back = (char *)ctx->stage[1];
+        for (uint32_t t = 0; t < count; ++t) {
+            const size_t b_bytes = (size_t)p.N[t] * 4u, o_bytes = (size_t)M * p.N[t] * 4u;
+            if (targets[t].bias) {
+                MI355Q_HIP(hipMemcpyAsync(in, targets[t].bias, b_bytes, hipMemcpyHostToDevice, ctx->stream),
+                           "bias upload");
+                p.bias[t] = (const float *)in;
+                in += b_bytes;
+            }
+            p.out[t] = (float *)back;
+            back += o_bytes;
+            if (targets[t].acc) {
+                p.acc[t] = (int32_t *)back;
+                back += o_bytes;
+            }
         }
-        p.out = (float *)ctx->stage[1];
-        p.acc = acc ? (int32_t *)((char *)ctx->stage[1] + o_bytes) : nullptr;
     }
     hipError_t launched;
     if (M > 32u)
-        launched = launch(ctx, w8a8_kernel<4>, dim3(weight->NT, (M + 63u) / 64u), dim3(256), 0, p);
+        launched = launch(ctx, w8a8_kernel<4>, dim3(tiles, (M + 63u) / 64u), dim3(256), 0, p);
     else if (M > 16u)
-        launched = launch(ctx, w8a8_kernel<2>, dim3(weight->NT, 1), dim3(256), 0, p);
+        launched = launch(ctx, w8a8_kernel<2>, dim3(tiles, 1), dim3(256), 0, p);
     else
-        launched = launch(ctx, w8a8_kernel<1>, dim3(weight->NT, 1), dim3(256), 0, p);
+        launched = launch(ctx, w8a8_kernel<1>, dim3(tiles, 1), dim3(256), 0, p);
     if (launched != hipSuccess) return fail_hip(launched, "w8a8 kernel launch", error, error_capacity);
     if (!device) {
-        MI355Q_HIP(hipMemcpyAsync(out, p.out, o_bytes, hipMemcpyDeviceToHost, ctx->stream),
-                   "output download");
-        if (acc)
-            MI355Q_HIP(hipMemcpyAsync(acc, p.acc, o_bytes, hipMemcpyDeviceToHost, ctx->stream),
-                       "accumulator download");
+        for (uint32_t t = 0; t < count; ++t) {
+            const size_t o_bytes = (size_t)M * p.N[t] * 4u;
+            MI355Q_HIP(hipMemcpyAsync(targets[t].out, p.out[t], o_bytes, hipMemcpyDeviceToHost, ctx->stream),
+                       "output download");
+            if (targets[t].acc)
+                MI355Q_HIP(hipMemcpyAsync(targets[t].acc, p.acc[t], o_bytes, hipMemcpyDeviceToHost,
+                                          ctx->stream),
+                           "accumulator download");
+        }
     }
     if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "w8a8_linear sync");
     return MI355Q_OK;
+}
+
+int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight, const int8_t *q,
+                       const float *x_scales, uint32_t M, const float *bias, float *out,
+                       int32_t *acc, uint32_t flags, char *error, size_t error_capacity)
+{
+    if (weight == nullptr || out == nullptr) {
+        set_error(error, error_capacity, "w8a8_linear: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    const mi355q_w8a8_target target = {weight, bias, out, acc};
+    return mi355q_w8a8_linear_multi(ctx, &target, 1, q, x_scales, M, flags, error, error_capacity);
 }
 
 }  // extern "C"

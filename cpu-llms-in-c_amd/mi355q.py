@@ -48,6 +48,10 @@ class Q4Target(_c.Structure):
     _fields_ = [("weight", _vp), ("y", _vp), ("residual", _vp)]
 
 
+class W8a8Target(_c.Structure):
+    _fields_ = [("weight", _vp), ("bias", _vp), ("out", _vp), ("acc", _vp)]
+
+
 class Q4Call(_c.Structure):
     _fields_ = [("x", _vp), ("M", _u32), ("x_dtype", _int), ("y_dtype", _int),
                 ("residual_dtype", _int), ("target_count", _u32), ("targets", Q4Target * 4),
@@ -112,6 +116,7 @@ SIGNATURES = {
     "mi355q_w8a8_weight_destroy": (None, [_vp]),
     "mi355q_quantize_i8": (_int, [_vp, _vp, _u32, _u32, _vp, _vp, _u32, *_err]),
     "mi355q_w8a8_linear": (_int, [_vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _u32, *_err]),
+    "mi355q_w8a8_linear_multi": (_int, [_vp, _vp, _u32, _vp, _vp, _u32, _u32, *_err]),
     "mi355q_synth_normal_f32": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_synth_normal_f16": (None, [_u64, _c.c_float, _sz, _vp]),
     "mi355q_quantize_q4_affine": (_int, [_vp, _u32, _u32, _int, _vp, _vp, _vp]),
@@ -454,6 +459,29 @@ class Context:
               _ptr(np.ascontiguousarray(x_scales, dtype=np.float32)), M, _ptr(bias), _ptr(out),
               _ptr(acc), W8A8_CHANNEL_MAJOR if channel_major else 0)
         return out, acc
+
+    def w8a8_linear_multi(self, weights, widths, q: np.ndarray, x_scales: np.ndarray, biases=None):
+        """One launch for up to four weights that share q: list of (out [M][N], acc [M][N])."""
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        M = q.shape[0]
+        biases = biases if biases is not None else [None] * len(weights)
+        biases = [None if b is None else np.ascontiguousarray(b, dtype=np.float32) for b in biases]
+        results = [(np.empty((M, N), dtype=np.float32), np.empty((M, N), dtype=np.int32)) for N in widths]
+        targets = (W8a8Target * len(weights))()
+        for slot, weight, bias, (out, acc) in zip(targets, weights, biases, results):
+            slot.weight, slot.bias, slot.out, slot.acc = weight, _ptr(bias), _ptr(out), _ptr(acc)
+        _call(self.lib.mi355q_w8a8_linear_multi, self.handle, targets, len(weights), _ptr(q),
+              _ptr(np.ascontiguousarray(x_scales, dtype=np.float32)), M, 0)
+        return results
+
+    def w8a8_linear_multi_device(self, weights, q_ptr: int, scales_ptr: int, M: int, bias_ptrs, out_ptrs,
+                                 acc_ptrs=None, asynchronous: bool = True):
+        targets = (W8a8Target * len(weights))()
+        for index, slot in enumerate(targets):
+            slot.weight, slot.bias, slot.out = weights[index], bias_ptrs[index], out_ptrs[index]
+            slot.acc = acc_ptrs[index] if acc_ptrs else None
+        _call(self.lib.mi355q_w8a8_linear_multi, self.handle, targets, len(weights), q_ptr, scales_ptr, M,
+              X_DEVICE | Y_DEVICE | (ASYNC if asynchronous else 0))
 
     def causal_q8_windows(self, x: np.ndarray, history, kernel: int, pairs: bool = False):
         """x [channels][length] fp32 -> (q [length][columns] int8, scales [length])."""

@@ -448,6 +448,21 @@ int mi355q_w8a8_linear(mi355q_context *ctx, const mi355q_w8a8_weight *weight,
                        const float *bias, float *out, int32_t *acc, uint32_t flags,
                        char *error, size_t error_capacity);
 
+/* Up to four weights of the same K against one quantized activation, in one
+ * launch: the reference quantizes a layer's normalised input once and multiplies
+ * it with the q, k and v weights in turn (minimindo_audio_encoder.c:400-403);
+ * here the three products share the launch as well.  Each target is one
+ * mi355q_w8a8_linear call's (weight, bias, out, acc). */
+typedef struct mi355q_w8a8_target {
+    const mi355q_w8a8_weight *weight;
+    const float *bias; /* [N] or NULL */
+    float *out;        /* [M][N] */
+    int32_t *acc;      /* [M][N] or NULL */
+} mi355q_w8a8_target;
+int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targets,
+                             uint32_t count, const int8_t *q, const float *x_scales,
+                             uint32_t M, uint32_t flags, char *error, size_t error_capacity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,3 +82,41 @@ def test_argument_errors(engine, gpu):
     with pytest.raises(engine.Mi355qError) as info:
         gpu.w8a8_prepare(rows, 16, 24)  # 24 is not a multiple of 16
     assert info.value.status == engine.ERROR_INVALID
+
+
+@pytest.mark.parametrize("M,K,widths", [(64, 1024, (4096, 4096, 4096)), (23, 560, (512, 100, 36, 512)),
+                                        (5, 48, (20, 16))])
+def test_projections_sharing_one_activation(engine, oracle, gpu, M, K, widths):
+    """q, k and v of an encoder layer multiply the same quantized activation
+    (minimindo_audio_encoder.c:400-403): one launch for all of them gives, per weight, the bits of
+    the single call (and of the oracle)."""
+    x = engine.synth_normal_f32(71, 1.0, M * K).reshape(M, K)
+    q, scales = oracle.quantize_i8(x)
+    rows = [engine.synth_w8_rows(80 + i, 0.02, N, K) for i, N in enumerate(widths)]
+    biases = [engine.synth_normal_f32(90 + i, 1.0, N) if i != 1 else None for i, N in enumerate(widths)]
+    weights = [gpu.w8a8_prepare(r, N, K) for r, N in zip(rows, widths)]
+    try:
+        print(f"w8a8 shared activation M={M} K={K} widths={widths}", flush=True)
+        results = gpu.w8a8_linear_multi(weights, widths, q, scales, biases)
+        for i, N in enumerate(widths):
+            out_ref, acc_ref = oracle.w8a8_linear(rows[i], N, K, q, scales, biases[i])
+            assert results[i][1].tobytes() == acc_ref.tobytes()
+            assert np.array_equal(results[i][0].view(np.uint32), out_ref.view(np.uint32))
+            single, _ = gpu.w8a8_linear(weights[i], N, q, scales, biases[i])
+            assert np.array_equal(single.view(np.uint32), results[i][0].view(np.uint32))
+    finally:
+        for weight in weights:
+            gpu.w8a8_destroy(weight)
+
+
+def test_shared_activation_needs_equal_columns(engine, gpu):
+    rows_a = engine.synth_w8_rows(1, 0.02, 32, 64)
+    rows_b = engine.synth_w8_rows(2, 0.02, 32, 128)
+    a, b = gpu.w8a8_prepare(rows_a, 32, 64), gpu.w8a8_prepare(rows_b, 32, 128)
+    try:
+        with pytest.raises(engine.Mi355qError) as caught:
+            gpu.w8a8_linear_multi([a, b], (32, 32), np.zeros((2, 64), np.int8), np.ones(2, np.float32))
+        assert caught.value.status == 2
+    finally:
+        gpu.w8a8_destroy(a)
+        gpu.w8a8_destroy(b)
