@@ -93,18 +93,34 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15u;
     const uint32_t kq = lane >> 4;
-    if (blockIdx.x >= p.columns) return;  // the grid is padded to a multiple of the XCD count
+    // The kernel arguments the first loads depend on are fetched in two batches (one wait each)
+    // instead of at their first uses, where every use would wait for its own fetch: a wave
+    // issues its first weight loads a microsecond earlier.
+    const uint32_t columns = p.columns, targets = p.targets, first1 = p.first_block[1],
+                   first2 = p.first_block[2], first3 = p.first_block[3];
+    const uint32_t T = p.T, K = p.K, slice_steps = p.slice_steps, chunk_steps = p.chunk_steps, rows = p.rows;
+    const int fuse_silu = p.fuse_silu;
+    const uint32_t *const ids = p.ids;
+    const _Float16 *const x = p.x;
+    asm volatile("" ::"s"(columns), "s"(targets), "s"(first1), "s"(first2), "s"(first3), "s"(T), "s"(K),
+                 "s"(slice_steps), "s"(chunk_steps), "s"(rows), "s"(fuse_silu), "s"(ids), "s"(x));
+    if (blockIdx.x >= columns) return;  // the grid is padded to a multiple of the XCD count
     uint32_t target = 0;
-#pragma unroll
-    for (uint32_t t = 1; t < kMaxTargets; ++t)
-        if (t < p.targets && blockIdx.x >= p.first_block[t]) target = t;
-    const uint32_t NT = p.NT[target], N = p.N[target], stride = p.stride[target];
+    if (1u < targets && blockIdx.x >= first1) target = 1;
+    if (2u < targets && blockIdx.x >= first2) target = 2;
+    if (3u < targets && blockIdx.x >= first3) target = 3;
+    const uint32_t NT = p.NT[target], N = p.N[target], stride = p.stride[target],
+                   first_block = p.first_block[target];
+    const uint4 *const codes_target = p.codes[target], *const codes_up = p.codes[1];
+    const uint2 *const meta_target = p.meta[target], *const meta_up = p.meta[1];
+    asm volatile("" ::"s"(NT), "s"(N), "s"(stride), "s"(first_block), "s"(codes_target), "s"(codes_up),
+                 "s"(meta_target), "s"(meta_up));
     // tiles per target and workgroup: TB, or TB/2 of each of the two fused targets
-    const uint32_t span_tiles = p.fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
-    const uint32_t tile0 = (blockIdx.x - p.first_block[target]) * span_tiles;
+    const uint32_t span_tiles = fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
+    const uint32_t tile0 = (blockIdx.x - first_block) * span_tiles;
 
     uint4 *xs = lds;                                                 // [chunk octets][MP]
-    float *red = (float *)(lds + (size_t)p.chunk_steps * 16u * MP);  // [W][TB][NJ][64]
+    float *red = (float *)(lds + (size_t)chunk_steps * 16u * MP);  // [W][TB][NJ][64]
 
     // per-tile record streams; a tile beyond the matrix re-reads the last tile
     // (its results are never stored)
@@ -112,22 +128,25 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint2 *meta_tile[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
-        const uint32_t slot_target = p.fuse_silu ? (uint32_t)tb / span_tiles : target;
+        // the fused pair's second half streams the second weight (up); everything else its target
+        const bool second = fuse_silu && (uint32_t)tb / span_tiles != 0u;
+        const uint4 *const codes_base = second ? codes_up : codes_target;
+        const uint2 *const meta_base = second ? meta_up : meta_target;
         uint32_t tile = tile0 + (uint32_t)tb % span_tiles;
         tile = tile < NT ? tile : NT - 1u;
-        if (p.ids != nullptr) {
+        if (ids != nullptr) {
             // gathered rows: lane (r, kq) streams row ids[16*tile + r] out of whichever tile holds
             // it (a slot or an id beyond the end re-reads a valid row; its result is not used)
             uint32_t slot = tile * kTileRows + r;
             slot = slot < N ? slot : N - 1u;
-            uint32_t row = p.ids[slot];
+            uint32_t row = ids[slot];
             row = row < p.matrix_rows ? row : p.matrix_rows - 1u;
-            codes_tile[tb] = p.codes[slot_target] + (size_t)(row / kTileRows) * 64u + kq * 16u + row % kTileRows;
-            meta_tile[tb] = p.meta[slot_target] + (size_t)(row / kTileRows) * 16u + row % kTileRows;
+            codes_tile[tb] = codes_base + (size_t)(row / kTileRows) * 64u + kq * 16u + row % kTileRows;
+            meta_tile[tb] = meta_base + (size_t)(row / kTileRows) * 16u + row % kTileRows;
             continue;
         }
-        codes_tile[tb] = p.codes[slot_target] + (size_t)tile * 64u + lane;
-        meta_tile[tb] = p.meta[slot_target] + (size_t)tile * 16u + r;
+        codes_tile[tb] = codes_base + (size_t)tile * 64u + lane;
+        meta_tile[tb] = meta_base + (size_t)tile * 16u + r;
     }
 
     floatx4 acc[TB];
@@ -137,10 +156,10 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const half8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
     const NibbleMasks masks = nibble_masks();
     const uint4 *xs_lane = xs + kq * MP + (r & (MP - 1));
-    const uint32_t slice_begin = blockIdx.y * p.slice_steps;
-    const uint32_t slice_end = slice_begin + p.slice_steps < p.T ? slice_begin + p.slice_steps : p.T;
-    for (uint32_t first = slice_begin; first < slice_end; first += p.chunk_steps) {
-        const uint32_t last = first + p.chunk_steps < slice_end ? first + p.chunk_steps : slice_end;
+    const uint32_t slice_begin = blockIdx.y * slice_steps;
+    const uint32_t slice_end = slice_begin + slice_steps < T ? slice_begin + slice_steps : T;
+    for (uint32_t first = slice_begin; first < slice_end; first += chunk_steps) {
+        const uint32_t last = first + chunk_steps < slice_end ? first + chunk_steps : slice_end;
         // this wave's steps in the chunk: first + wave + i*W, i < count
         const uint32_t span = last - first;
         const uint32_t count = wave < span ? (span - wave + W - 1u) / W : 0u;
@@ -160,7 +179,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         auto issue_clamped = [&](uint32_t i, StepData<TB> &slot) {
             const uint32_t clamped = i < count ? i : (count ? count - 1u : 0u);
             uint32_t step = step0 + clamped * W;
-            step = step < p.T ? step : p.T - 1u;
+            step = step < T ? step : T - 1u;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
                 slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * stride * 64u);
@@ -168,21 +187,26 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             }
         };
         // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
-        // The activation loads go out first (they come back from L2 quickly),
-        // then the first D weight steps; the LDS stores wait for the former only.
+        // The activation loads go out first (they come back from L2 quickly), then, without
+        // a wait in between, the first D weight steps; loads return in order, so the LDS
+        // stores wait for the former only.
         constexpr int SB = MP == 1 ? 5 : 10;  // fetches in flight per thread: one L2 round trip for most slices
         const uint32_t octets = span * 16u;
         const uint32_t items = octets * MP;
         auto stage_fetch = [&](uint32_t index) {
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
-            if (index < items) {
-                // consecutive threads fill consecutive LDS slots (no bank conflicts); each
-                // activation row still contributes runs of 64/MP adjacent octets
-                const uint32_t mrow = index % MP, o = index / MP;
-                const uint32_t k = first * kStepColumns + o * 8u;
-                if (mrow < p.rows && k < p.K) v = *(const uint4 *)(p.x + (size_t)mrow * p.K + k);
-            }
-            return v;
+            // consecutive threads fill consecutive LDS slots (no bank conflicts); each
+            // activation row still contributes runs of 64/MP adjacent octets.  The load is
+            // unconditional (a slot with nothing to fetch reads the first octet of x and
+            // becomes zero afterwards): no branch, so no wait, between the fetches.
+            const uint32_t mrow = index % MP, o = index / MP;
+            const uint32_t k = first * kStepColumns + o * 8u;
+            const bool live = index < items && mrow < rows && k < K;
+            const uint4 v = *(const uint4 *)(x + (live ? (size_t)mrow * K + k : (size_t)0));
+            // a mask the compiler cannot see through: a select here would be turned back into
+            // a branch around the load
+            uint32_t keep = live ? 0xffffffffu : 0u;
+            asm volatile("" : "+v"(keep));
+            return make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
         };
         auto stage_store = [&](uint32_t index, const uint4 &v) {
             if (index < items) xs[index] = v;
