@@ -124,14 +124,18 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 
     // per-tile record streams; a tile beyond the matrix re-reads the last tile
     // (its results are never stored)
-    const uint4 *codes_tile[TB];
-    const uint2 *meta_tile[TB];
+    // A record's address = a base that is the same for the whole wave (weight + step, 64-bit,
+    // scalar arithmetic) + a byte offset per lane that never changes (32 bits: a matrix's
+    // tiles of one step span less than 4 GiB): the loads need no vector address arithmetic.
+    const char *codes_base[TB];
+    const char *meta_base[TB];
+    uint32_t codes_lane[TB], meta_lane[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
         // the fused pair's second half streams the second weight (up); everything else its target
         const bool second = fuse_silu && (uint32_t)tb / span_tiles != 0u;
-        const uint4 *const codes_base = second ? codes_up : codes_target;
-        const uint2 *const meta_base = second ? meta_up : meta_target;
+        codes_base[tb] = (const char *)(second ? codes_up : codes_target);
+        meta_base[tb] = (const char *)(second ? meta_up : meta_target);
         uint32_t tile = tile0 + (uint32_t)tb % span_tiles;
         tile = tile < NT ? tile : NT - 1u;
         if (ids != nullptr) {
@@ -141,13 +145,14 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             slot = slot < N ? slot : N - 1u;
             uint32_t row = ids[slot];
             row = row < p.matrix_rows ? row : p.matrix_rows - 1u;
-            codes_tile[tb] = codes_base + (size_t)(row / kTileRows) * 64u + kq * 16u + row % kTileRows;
-            meta_tile[tb] = meta_base + (size_t)(row / kTileRows) * 16u + row % kTileRows;
+            codes_lane[tb] = ((row / kTileRows) * 64u + kq * 16u + row % kTileRows) * (uint32_t)sizeof(uint4);
+            meta_lane[tb] = ((row / kTileRows) * 16u + row % kTileRows) * (uint32_t)sizeof(uint2);
             continue;
         }
-        codes_tile[tb] = codes_base + (size_t)tile * 64u + lane;
-        meta_tile[tb] = meta_base + (size_t)tile * 16u + r;
+        codes_lane[tb] = (tile * 64u + lane) * (uint32_t)sizeof(uint4);
+        meta_lane[tb] = (tile * 16u + r) * (uint32_t)sizeof(uint2);
     }
+    const size_t codes_step = (size_t)stride * 64u * sizeof(uint4), meta_step = (size_t)stride * 16u * sizeof(uint2);
 
     floatx4 acc[TB];
 #pragma unroll
@@ -172,8 +177,18 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             const uint32_t step = step0 + i * W;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * stride * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * stride * 16u);
+                // the step's base stays in scalar registers (the empty asm pins it there), so the
+                // load takes it as its scalar base and the lane offset as its vector offset
+                uint64_t codes_at = (uint64_t)(codes_base[tb] + step * codes_step);
+                uint64_t meta_at = (uint64_t)(meta_base[tb] + step * meta_step);
+                asm volatile("" : "+s"(codes_at), "+s"(meta_at));
+                typedef const __attribute__((address_space(1))) char *global_bytes;
+                const u32x4 q = __builtin_nontemporal_load(
+                    (const __attribute__((address_space(1))) u32x4 *)((global_bytes)codes_at + codes_lane[tb]));
+                const u32x2 m = __builtin_nontemporal_load(
+                    (const __attribute__((address_space(1))) u32x2 *)((global_bytes)meta_at + meta_lane[tb]));
+                slot.q[tb] = make_uint4(q.x, q.y, q.z, q.w);
+                slot.m[tb] = make_uint2(m.x, m.y);
             }
         };
         auto issue_clamped = [&](uint32_t i, StepData<TB> &slot) {
@@ -182,8 +197,18 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             step = step < T ? step : T - 1u;
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
-                slot.q[tb] = load_stream(codes_tile[tb] + (size_t)step * stride * 64u);
-                slot.m[tb] = load_stream(meta_tile[tb] + (size_t)step * stride * 16u);
+                // the step's base stays in scalar registers (the empty asm pins it there), so the
+                // load takes it as its scalar base and the lane offset as its vector offset
+                uint64_t codes_at = (uint64_t)(codes_base[tb] + step * codes_step);
+                uint64_t meta_at = (uint64_t)(meta_base[tb] + step * meta_step);
+                asm volatile("" : "+s"(codes_at), "+s"(meta_at));
+                typedef const __attribute__((address_space(1))) char *global_bytes;
+                const u32x4 q = __builtin_nontemporal_load(
+                    (const __attribute__((address_space(1))) u32x4 *)((global_bytes)codes_at + codes_lane[tb]));
+                const u32x2 m = __builtin_nontemporal_load(
+                    (const __attribute__((address_space(1))) u32x2 *)((global_bytes)meta_at + meta_lane[tb]));
+                slot.q[tb] = make_uint4(q.x, q.y, q.z, q.w);
+                slot.m[tb] = make_uint2(m.x, m.y);
             }
         };
         // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
