@@ -119,13 +119,14 @@ def weights_digest(host, shapes):
     return digest.hexdigest()
 
 
-def cpu_baseline(oracle, shapes, host, M, meta_kind, repeats=5):
-    """The oracle's reference-faithful flavour (fp32, k order) on all host threads."""
+def cpu_baseline(oracle, shapes, host, M, meta_kind, budget_s=10.0):
+    """The oracle's reference-faithful flavour (fp32, k order) on all host threads: passes over
+    the layer for about `budget_s` seconds (at least 5, at most 200), the median taken."""
     threads = min(os.cpu_count() or 1, 16)
     os.environ.setdefault("OMP_NUM_THREADS", str(threads))
     total_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
-    times = []
-    for rep in range(repeats + 1):
+    times, repeats, rep = [], 5, 0
+    while rep < repeats + 1:
         t0 = time.perf_counter()
         for name, N, K in shapes:
             quants, meta_a, meta_b = host[name]
@@ -133,6 +134,9 @@ def cpu_baseline(oracle, shapes, host, M, meta_kind, repeats=5):
                              M, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=threads)
         if rep:
             times.append(time.perf_counter() - t0)
+        if rep == 1:  # the first pass warms up; the second sizes the sample
+            repeats = max(5, min(200, int(budget_s / max(times[0], 1e-4))))
+        rep += 1
     median = sorted(times)[len(times) // 2]
     t0 = time.perf_counter()  # the reference's deployment width: four threads (one pass)
     for name, N, K in shapes:
