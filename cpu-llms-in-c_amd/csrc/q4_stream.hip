@@ -586,23 +586,35 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         const uint32_t want = (8u * cus + groups - 1) / groups;
         shape.waves = want <= 2u ? 2 : want <= 6u ? 4 : 8;
         if (NT_total <= cus + cus / 2u && T >= 96u) {
-            // few tiles with long rows (the 27B down projection): four K slices of pairs of
-            // tiles keep more loads in flight than eight waves on one tile each
+            // few tiles with long rows (the 27B down projection): K slices of pairs of tiles
+            // keep more loads in flight than eight waves on one tile each.  With more tiles
+            // than compute units, as many slices as keep the workgroups within two per
+            // compute unit (down: three slices of 160 pairs, 480 workgroups, 13.5 us against
+            // 14.5 with four slices, where half of the compute units get a third workgroup)
             shape.tb = 2;
             shape.waves = 4;
-            slices = 4;
+            slices = NT_total > cus ? 2u * cus / ((NT_total + 1u) / 2u) : 4u;
+        } else if (NT_total > cus && NT_total <= cus + cus / 2u) {
+            // a few more tiles than compute units (the 27B o projection, 320 tiles): one
+            // workgroup per tile gives a quarter of the compute units two workgroups and the
+            // rest one; pairs of tiles leave every compute unit at most one workgroup of
+            // eight waves (7.55 -> 7.28 us)
+            shape.tb = 2;
+            shape.waves = 8;
         }
     } else {
         // every workgroup copies its activation rows from L2 into LDS: two tiles per
         // workgroup halve that traffic.  Matrices with few tiles and long rows are cut in
         // slices (of 32 steps or more: adding the slices costs about as much as a few
-        // steps) until some 2.5 workgroups per compute unit exist.
+        // steps) until some 2 to 2.5 workgroups per compute unit exist.
         shape.tb = NT_total >= cus ? 2 : 1;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
-        slices = (5u * cus / 2u + groups / 2u) / groups;
+        // (up to four rows two workgroups per compute unit are enough: down at M = 2 and 4 is
+        // 6-8 % faster in three slices than in four)
+        slices = mp <= 4 ? 2u * cus / groups : (5u * cus / 2u + groups / 2u) / groups;
         if (slices > T / 32u) slices = T / 32u;
         choose_cuts(shape, T, slices);
-        const uint32_t want = (16u * cus + groups * shape.slices - 1) / (groups * shape.slices);
+        const uint32_t want = 16u * cus / (groups * shape.slices);
         shape.waves = want <= 2u ? 2 : want <= 8u ? 4 : 8;
     }
     // "TB,DEPTH,WAVES[,SLICES]" for experiments
