@@ -29,8 +29,23 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
+#include <utility>
 
 namespace mi355q {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
+// compile-time constant in the body
+template <int... I, class F>
+__device__ __forceinline__ void stream_static_for_impl(std::integer_sequence<int, I...>, F &&f)
+{
+    (f(std::integral_constant<int, I>()), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    stream_static_for_impl(std::make_integer_sequence<int, N>(), f);
+}
 
 struct StreamParams {
     // up to kMaxTargets weights share the activations; workgroups
@@ -119,8 +134,21 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint32_t span_tiles = fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
     const uint32_t tile0 = (blockIdx.x - first_block) * span_tiles;
 
-    uint4 *xs = lds;                                                 // [chunk octets][MP]
-    float *red = (float *)(lds + (size_t)chunk_steps * 16u * MP);  // [W][TB][NJ][64]
+    // LDS: every wave owns R slots of activations, one per step it has in flight (a step's
+    // activations are read by the one wave that takes the step: nothing is shared, so there is
+    // no barrier and no copy through registers; the loads write LDS directly), then the area
+    // where the waves' partial sums meet.
+    constexpr bool AHEAD = MP >= 4;
+    constexpr int R = AHEAD ? D + 1 : D;
+    constexpr int XI = MP >= 4 ? MP / 4 : 1;  // 64-lane loads that fill one slot
+    constexpr uint32_t SLAB = 64u * XI;       // 16-byte entries per slot: [octet][row], padded to whole loads
+    constexpr int S = XI + 2 * TB;            // vector memory operations per step of a wave
+    static_assert(S * (D + 1) <= 63, "the load counter has six bits");
+    uint4 *const ring_x = lds + (size_t)wave * (R * SLAB);
+    float *red = (float *)(lds + (size_t)W * (R * SLAB));  // [W][TB][NJ][64]
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr)ring_x);
+
 
     // per-tile record streams; a tile beyond the matrix re-reads the last tile
     // (its results are never stored)
@@ -154,27 +182,56 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     }
     const size_t codes_step = (size_t)stride * 64u * sizeof(uint4), meta_step = (size_t)stride * 16u * sizeof(uint2);
 
+    // where lane l reads the activations it brings into a slot: entry e = l + 64 b of the slot
+    // is (octet e / MP, row e % MP).  Rows beyond the last repeat it and octets beyond the
+    // step's sixteen repeat the last (entries nobody reads, or rows nobody stores).
+    uint32_t x_lane[XI], x_lane_tail[XI];
+#pragma unroll
+    for (int b = 0; b < XI; ++b) {
+        const uint32_t e = lane + 64u * b;
+        uint32_t o = e / MP, mrow = e % MP;
+        o = o < 16u ? o : 15u;
+        mrow = mrow < rows ? mrow : rows - 1u;
+        x_lane[b] = (mrow * K + o * 8u) * (uint32_t)sizeof(_Float16);
+        // K is a multiple of 64: when it is an odd one, the upper half of the last step does not
+        // exist (its codes and metadata are zero); the lane reads the lower half again
+        x_lane_tail[b] = x_lane[b] - (o >= 8u ? 64u * (uint32_t)sizeof(_Float16) : 0u);
+    }
+    const bool odd_tail = (K % kStepColumns) != 0u;
+
     floatx4 acc[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) acc[tb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     const floatx4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     const half8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
     const NibbleMasks masks = nibble_masks();
-    const uint4 *xs_lane = xs + kq * MP + (r & (MP - 1));
     const uint32_t slice_begin = blockIdx.y * slice_steps;
     const uint32_t slice_end = slice_begin + slice_steps < T ? slice_begin + slice_steps : T;
-    for (uint32_t first = slice_begin; first < slice_end; first += chunk_steps) {
-        const uint32_t last = first + chunk_steps < slice_end ? first + chunk_steps : slice_end;
-        // this wave's steps in the chunk: first + wave + i*W, i < count
-        const uint32_t span = last - first;
+    {
+        // this wave's steps in the slice: slice_begin + wave + i*W, i < count
+        const uint32_t span = slice_end - slice_begin;
         const uint32_t count = wave < span ? (span - wave + W - 1u) / W : 0u;
-        const uint32_t step0 = first + wave;
+        const uint32_t step0 = slice_begin + wave;
 
-        // In the main loop every step is paired with one refill, unconditionally, so the
-        // number of loads in flight is known at compile time and each step waits only for
-        // its own data; only the first D loads (a wave may own fewer steps) clamp.
-        auto issue = [&](uint32_t i, StepData<TB> &slot) {
-            const uint32_t step = step0 + i * W;
+        // One step's fetch = XI loads of activations straight into the LDS slot, then codes and
+        // metadata of each tile into registers: S vector memory operations, always in this
+        // order.  Loads complete in order, so "at most S*n operations outstanding" means
+        // "everything up to the n-th newest fetch has landed".
+        auto fetch = [&](uint32_t step, auto slot_c, StepData<TB> &slot) {
+            constexpr uint32_t slot_bytes = decltype(slot_c)::value * SLAB * (uint32_t)sizeof(uint4);
+            uint64_t x_at = (uint64_t)((const char *)x + (size_t)step * (kStepColumns * sizeof(_Float16)));
+            asm volatile("" : "+s"(x_at));
+            const bool tail_step = odd_tail && step + 1u == T;
+#pragma unroll
+            for (int b = 0; b < XI; ++b) {
+                const uint32_t offset = tail_step ? x_lane_tail[b] : x_lane[b];
+                // the slot was last read by the step consumed before this fetch: those LDS reads
+                // have returned before the write can land (wait for them all the same)
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                             :
+                             : "v"(offset), "s"(x_at), "s"(lds_wave + slot_bytes + 1024u * (uint32_t)b)
+                             : "memory");
+            }
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
                 // the step's base stays in scalar registers (the empty asm pins it there), so the
@@ -191,77 +248,36 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 slot.m[tb] = make_uint2(m.x, m.y);
             }
         };
-        auto issue_clamped = [&](uint32_t i, StepData<TB> &slot) {
+        // In the main loop every step is paired with one refill, unconditionally, so the
+        // number of loads in flight is known at compile time and each step waits only for
+        // its own data; only the first D fetches (a wave may own fewer steps) clamp.
+        auto issue = [&](uint32_t i, auto slot_c, StepData<TB> &slot) { fetch(step0 + i * W, slot_c, slot); };
+        auto issue_clamped = [&](uint32_t i, auto slot_c, StepData<TB> &slot) {
             const uint32_t clamped = i < count ? i : (count ? count - 1u : 0u);
             uint32_t step = step0 + clamped * W;
             step = step < T ? step : T - 1u;
-#pragma unroll
-            for (int tb = 0; tb < TB; ++tb) {
-                // the step's base stays in scalar registers (the empty asm pins it there), so the
-                // load takes it as its scalar base and the lane offset as its vector offset
-                uint64_t codes_at = (uint64_t)(codes_base[tb] + step * codes_step);
-                uint64_t meta_at = (uint64_t)(meta_base[tb] + step * meta_step);
-                asm volatile("" : "+s"(codes_at), "+s"(meta_at));
-                typedef const __attribute__((address_space(1))) char *global_bytes;
-                const u32x4 q = __builtin_nontemporal_load(
-                    (const __attribute__((address_space(1))) u32x4 *)((global_bytes)codes_at + codes_lane[tb]));
-                const u32x2 m = __builtin_nontemporal_load(
-                    (const __attribute__((address_space(1))) u32x2 *)((global_bytes)meta_at + meta_lane[tb]));
-                slot.q[tb] = make_uint4(q.x, q.y, q.z, q.w);
-                slot.m[tb] = make_uint2(m.x, m.y);
-            }
+            fetch(step, slot_c, slot);
         };
-        // ---- activations of this chunk into LDS: [octet][row], 16 bytes each.
-        // The activation loads go out first (they come back from L2 quickly), then, without
-        // a wait in between, the first D weight steps; loads return in order, so the LDS
-        // stores wait for the former only.
-        constexpr int SB = MP == 1 ? 5 : 10;  // fetches in flight per thread: one L2 round trip for most slices
-        const uint32_t octets = span * 16u;
-        const uint32_t items = octets * MP;
-        auto stage_fetch = [&](uint32_t index) {
-            // consecutive threads fill consecutive LDS slots (no bank conflicts); each
-            // activation row still contributes runs of 64/MP adjacent octets.  The load is
-            // unconditional (a slot with nothing to fetch reads the first octet of x and
-            // becomes zero afterwards): no branch, so no wait, between the fetches.
-            const uint32_t mrow = index % MP, o = index / MP;
-            const uint32_t k = first * kStepColumns + o * 8u;
-            const bool live = index < items && mrow < rows && k < K;
-            const uint4 v = *(const uint4 *)(x + (live ? (size_t)mrow * K + k : (size_t)0));
-            // a mask the compiler cannot see through: a select here would be turned back into
-            // a branch around the load
-            uint32_t keep = live ? 0xffffffffu : 0u;
-            asm volatile("" : "+v"(keep));
-            return make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
+        // waits until at most `fetches` whole fetches are outstanding
+        auto wait_fetches = [&](auto fetches_c) {
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(fetches_c)::value * S) : "memory");
         };
-        auto stage_store = [&](uint32_t index, const uint4 &v) {
-            if (index < items) xs[index] = v;
+        auto wait_fetches_counted = [&](uint32_t fetches) {
+            static_for<D + 1>([&](auto n_c) {
+                if (fetches == (uint32_t) decltype(n_c)::value) wait_fetches(n_c);
+            });
+            if (fetches > (uint32_t)D) wait_fetches(std::integral_constant<int, D>());
         };
-        uint4 staged[SB];
-#pragma unroll
-        for (int b = 0; b < SB; ++b) staged[b] = stage_fetch(threadIdx.x + b * 64u * W);
 
         // With four activation rows or more the arithmetic of a step is long enough to matter:
-        // one more register set than steps in flight lets a step's refill go out before the
-        // step is worked on instead of after (gate|up at M = 8: 9 %; at M = 1 it costs 1 %).
-        constexpr bool AHEAD = MP >= 4;
-        constexpr int R = AHEAD ? D + 1 : D;
+        // one more register set (and LDS slot) than steps in flight lets a step's refill go out
+        // before the step is worked on instead of after (gate|up at M = 8: 9 %; at M = 1 it
+        // costs 1 %).
         StepData<TB> ring[R];
-#pragma unroll
-        for (int u = 0; u < D; ++u) issue_clamped(u, ring[u]);
+        static_for<D>([&](auto u_c) { issue_clamped(decltype(u_c)::value, u_c, ring[decltype(u_c)::value]); });
 
-        if (first > slice_begin) __syncthreads();  // everyone is done with the previous chunk
-#pragma unroll
-        for (int b = 0; b < SB; ++b) stage_store(threadIdx.x + b * 64u * W, staged[b]);
-        for (uint32_t base = threadIdx.x + SB * 64u * W; base < items; base += SB * 64u * W) {
-#pragma unroll
-            for (int b = 0; b < SB; ++b) staged[b] = stage_fetch(base + b * 64u * W);
-#pragma unroll
-            for (int b = 0; b < SB; ++b) stage_store(base + b * 64u * W, staged[b]);
-        }
-        __syncthreads();
-
-        auto consume = [&](uint32_t i, const StepData<TB> &slot) {
-            const uint4 *xp = xs_lane + (size_t)(wave + i * W) * 16u * MP;
+        auto consume = [&](auto slot_c, const StepData<TB> &slot) {
+            const uint4 *xp = ring_x + decltype(slot_c)::value * SLAB + kq * MP + (r & (MP - 1));
             const half8 a0 = __builtin_bit_cast(half8, xp[0]);
             const half8 a1 = __builtin_bit_cast(half8, xp[4 * MP]);
             const half8 a2 = __builtin_bit_cast(half8, xp[8 * MP]);
@@ -296,50 +312,73 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 }
             }
         };
+        // fetches issued so far: steps 0 .. issued-1 of this wave (the first D always, clamped)
         if constexpr (AHEAD) {
             // main part: whole rounds over the R register sets whose refills all exist; step i
             // lives in set i % R, and its refill (step i + D) goes to the set freed by step i - 1
             const uint32_t main_end = count > (uint32_t)D ? (count - D) / R * R : 0u;
             for (uint32_t base = 0; base < main_end; base += R) {
-#pragma unroll
-                for (int u = 0; u < R; ++u) {
-                    issue(base + u + D, ring[(u + D) % R]);
-                    consume(base + u, ring[u]);
-                }
+                static_for<R>([&](auto u_c) {
+                    constexpr int u = decltype(u_c)::value;
+                    constexpr int to = (u + D) % R;
+                    issue(base + u + D, std::integral_constant<int, to>(), ring[to]);
+                    wait_fetches(std::integral_constant<int, D>());
+                    consume(u_c, ring[u]);
+                });
             }
             // the last (fewer than R + D) steps: refill only while steps remain
-#pragma unroll
-            for (int t = 0; t < R + D - 1; ++t) {
+            uint32_t issued = main_end + D;
+            static_for<R + D - 1>([&](auto t_c) {
+                constexpr int t = decltype(t_c)::value;
                 const uint32_t i = main_end + t;
                 if (i < count) {
-                    if (i + D < count) issue(i + D, ring[(t + D) % R]);
-                    consume(i, ring[t % R]);
+                    if (i + D < count) {
+                        constexpr int to = (t + D) % R;
+                        issue(i + D, std::integral_constant<int, to>(), ring[to]);
+                        issued = i + D + 1u;
+                    }
+                    wait_fetches_counted(issued - 1u - i);
+                    consume(std::integral_constant<int, t % R>(), ring[t % R]);
                 }
-            }
+            });
         } else {
             // main part: whole groups of D steps whose refills all exist
             const uint32_t main_end = count > (uint32_t)D ? (count - D) / D * D : 0u;
             for (uint32_t base = 0; base < main_end; base += D) {
-#pragma unroll
-                for (int u = 0; u < D; ++u) {
-                    consume(base + u, ring[u]);
-                    issue(base + u + D, ring[u]);  // refill the slot just consumed
-                }
+                static_for<D>([&](auto u_c) {
+                    constexpr int u = decltype(u_c)::value;
+                    wait_fetches(std::integral_constant<int, D - 1>());
+                    consume(u_c, ring[u]);
+                    issue(base + u + D, u_c, ring[u]);  // refill the slot just consumed
+                });
             }
             // the last (at most 2D - 1) steps: refill only while steps remain, then drain
-#pragma unroll
-            for (int u = 0; u < D; ++u) {
+            uint32_t issued = main_end + D;
+            static_for<D>([&](auto u_c) {
+                constexpr int u = decltype(u_c)::value;
                 const uint32_t i = main_end + u;
                 if (i < count) {
-                    consume(i, ring[u]);
-                    if (i + D < count) issue(i + D, ring[u]);
+                    wait_fetches_counted(issued - 1u - i);
+                    consume(u_c, ring[u]);
+                    if (i + D < count) {
+                        issue(i + D, u_c, ring[u]);
+                        issued = i + D + 1u;
+                    }
                 }
-            }
-#pragma unroll
-            for (int u = 0; u < D; ++u)
-                if (main_end + D + u < count) consume(main_end + D + u, ring[u]);
+            });
+            static_for<D>([&](auto u_c) {
+                constexpr int u = decltype(u_c)::value;
+                const uint32_t i = main_end + D + u;
+                if (i < count) {
+                    wait_fetches_counted(issued - 1u - i);
+                    consume(u_c, ring[u]);
+                }
+            });
         }
+        // no load may still be on its way into LDS when the workgroup gives its LDS back
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+
 
     // ---- add the waves' partial sums in wave order, then store
 #pragma unroll
@@ -511,10 +550,15 @@ struct StreamShape {
     uint32_t slices, slice_steps, chunk_steps;
 };
 
-static size_t stream_lds_bytes(int mp, int tb, int waves, uint32_t chunk_steps)
+// every wave's ring of activation slots (one more than its steps in flight from four rows on;
+// a slot holds a step's 16 octets of every row, padded to whole 64-lane loads), then the
+// partial sums of all waves
+static size_t stream_lds_bytes(int mp, int tb, int depth, int waves)
 {
     const int nj = mp < 4 ? mp : 4;
-    return (size_t)chunk_steps * 256u * mp + (size_t)waves * tb * nj * 256u;
+    const int slots = mp >= 4 ? depth + 1 : depth;
+    const size_t slab = 1024u * (size_t)(mp >= 4 ? mp / 4 : 1);
+    return (size_t)waves * slots * slab + (size_t)waves * tb * nj * 256u;
 }
 
 template <int MP, int TB, int D, int W>
@@ -525,7 +569,7 @@ static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
         blocks = (p.NT[0] + (TB > 1 ? TB / 2 : 1) - 1) / (TB > 1 ? TB / 2 : 1);
     else
         for (uint32_t t = 0; t < p.targets; ++t) blocks += (p.NT[t] + TB - 1) / TB;
-    const size_t lds = stream_lds_bytes(MP, TB, W, p.chunk_steps);
+    const size_t lds = stream_lds_bytes(MP, TB, D, W);
     StreamParams q = p;
     q.columns = blocks;
     // slices added in the kernel: the slices of one column must land on one XCD, which they do
@@ -560,7 +604,7 @@ static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const
 // (walked by one workgroup) whose activations take at most 40 KiB of LDS.
 static void choose_cuts(StreamShape &shape, uint32_t T, uint32_t slices)
 {
-    const uint32_t max_steps = (40u * 1024u) / (256u * (uint32_t)shape.mp);
+    const uint32_t max_steps = T;  // the activations pass through per-wave slots: no chunks
     slices = slices < 1u ? 1u : slices > T ? T : slices;
     shape.slice_steps = (T + slices - 1) / slices;
     shape.slices = (T + shape.slice_steps - 1) / shape.slice_steps;
@@ -629,6 +673,8 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
     }
     choose_cuts(shape, T, slices);
     while (shape.waves > 2 && (uint32_t)shape.waves > shape.chunk_steps) shape.waves /= 2;
+    while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
+        shape.waves /= 2;
     return shape;
 }
 
@@ -671,6 +717,8 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         tiles += subset ? (a.row_count + kTileRows - 1) / kTileRows : a.targets[t].w->NT;
     StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
     if (a.fuse_silu && shape.tb != 2 && shape.tb != 4) shape.tb = 2;  // gate and up tiles pair up
+    while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
+        shape.waves /= 2;
     uint32_t block = 0;
     for (uint32_t t = 0; t < a.count; ++t) {
         const Q4Device &w = *a.targets[t].w;
@@ -715,7 +763,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.residual_is_bias = a.residual_is_bias;
     p.meta_bf16 = first.meta_kind == MI355Q_META_BF16_PLANES;
 
-    const size_t lds = stream_lds_bytes(mp, shape.tb, shape.waves, shape.chunk_steps);
+    const size_t lds = stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves);
     if (lds + 64u > 64u * 1024u) {  // a few bytes of static LDS besides
         set_error(error, error_capacity, "q4 stream kernel: %zu bytes of LDS needed (K=%u, rows=%u)",
                   lds, first.K, rows);
