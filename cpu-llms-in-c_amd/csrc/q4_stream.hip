@@ -620,46 +620,36 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
     shape.tb = 1;
     shape.depth = 2;
     uint32_t slices = 1;
-    if (mp == 1) {
-        // two to three thousand waves with two steps of loads in flight each keep HBM busy
-        // without queueing (gate|up: 2176 waves of 20 steps against 4352 of 10: 1 % faster); with a thousand tiles or more a workgroup takes two or four (fewer
-        // copies of x into LDS and fewer workgroups to start for the same number of waves);
-        // more waves per workgroup when there are few tiles
-        shape.tb = NT_total >= 32u * cus ? 4 : NT_total >= 4u * cus ? 2 : 1;  // four: the LM head
+    if (mp <= 2) {
+        // One or two activation rows: a step's activations are a quarter or half of a 64-lane
+        // load, so nothing is gained by sharing them between tiles; one tile per workgroup and
+        // many workgroups stream best (gate|up at M = 1: 2176 workgroups of four waves 19.3 us,
+        // 1088 pairs of tiles 20.2-20.5; at M = 2 20.1 against 23.4), eight waves when the
+        // tiles are few (q|k|v 7.3 against 8.15 us with four).  Only a matrix with tens of
+        // thousands of tiles (the LM head) takes two or four per workgroup, two waves each.
+        shape.tb = NT_total >= 32u * cus ? 4 : NT_total >= 12u * cus ? 2 : 1;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
-        const uint32_t want = (8u * cus + groups - 1) / groups;
-        shape.waves = want <= 2u ? 2 : want <= 6u ? 4 : 8;
+        shape.waves = shape.tb > 1 ? 2 : groups <= 3u * cus ? 8 : 4;
         if (NT_total <= cus + cus / 2u && T >= 96u) {
-            // few tiles with long rows (the 27B down projection): K slices of pairs of tiles
-            // keep more loads in flight than eight waves on one tile each.  With more tiles
-            // than compute units, as many slices as keep the workgroups within two per
-            // compute unit (down: three slices of 160 pairs, 480 workgroups, 13.5 us against
-            // 14.5 with four slices, where half of the compute units get a third workgroup)
-            shape.tb = 2;
+            // few tiles with long rows (the 27B down projection): K slices keep more loads in
+            // flight than eight waves on a whole row.  With more tiles than compute units,
+            // three slices of four waves (down: 12.9-13.2 us; two slices 14.5, four 13.6,
+            // pairs of tiles in three slices 13.6-13.8)
             shape.waves = 4;
-            slices = NT_total > cus ? 2u * cus / ((NT_total + 1u) / 2u) : 4u;
-        } else if (NT_total > cus && NT_total <= cus + cus / 2u) {
-            // a few more tiles than compute units (the 27B o projection, 320 tiles): one
-            // workgroup per tile gives a quarter of the compute units two workgroups and the
-            // rest one; pairs of tiles leave every compute unit at most one workgroup of
-            // eight waves (7.55 -> 7.28 us)
-            shape.tb = 2;
-            shape.waves = 8;
+            slices = NT_total > cus ? 3u : 4u;
         }
     } else {
-        // every workgroup copies its activation rows from L2 into LDS: two tiles per
-        // workgroup halve that traffic.  Matrices with few tiles and long rows are cut in
+        // With four rows or more a step's activations are whole loads (one per four rows), which
+        // two tiles per workgroup share.  Matrices with few tiles and long rows are cut in
         // slices (of 32 steps or more: adding the slices costs about as much as a few
-        // steps) until some 2 to 2.5 workgroups per compute unit exist.
+        // steps) until some two workgroups per compute unit exist.
         shape.tb = NT_total >= cus ? 2 : 1;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
-        // (up to four rows two workgroups per compute unit are enough: down at M = 2 and 4 is
-        // 6-8 % faster in three slices than in four)
-        slices = mp <= 4 ? 2u * cus / groups : (5u * cus / 2u + groups / 2u) / groups;
+        slices = 2u * cus / groups;
         if (slices > T / 32u) slices = T / 32u;
         choose_cuts(shape, T, slices);
         const uint32_t want = 16u * cus / (groups * shape.slices);
-        shape.waves = want <= 2u ? 2 : want <= 8u ? 4 : 8;
+        shape.waves = want <= 2u ? 2 : want < 8u ? 4 : 8;
     }
     // "TB,DEPTH,WAVES[,SLICES]" for experiments
     const char *force = getenv("MI355Q_Q4_STREAM");
