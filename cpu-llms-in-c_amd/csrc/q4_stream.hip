@@ -16,13 +16,14 @@
 // (a fixed order: results do not depend on timing).  Nothing is shared between
 // workgroups.
 //
-// The workgroup copies the activations of its columns into LDS (laid out
-// [octet of columns][row], so a wave's fragment reads are contiguous) and every
-// wave reads its steps from there.  With several activation rows that copy is as
-// large as the weights a tile brings, so a workgroup then takes two tiles, long
-// rows are cut in slices over workgroups (fp32 partial sums, added in slice order
-// by whichever workgroup of the column finishes last), and a slice that still
-// overflows LDS is walked in chunks.
+// A step's activations are needed by the one wave that takes the step, so every
+// wave brings them in itself, with the step's weights: loads that write LDS
+// directly (no registers in between) fill a slot of the wave's own small ring,
+// laid out [octet of columns][row] so that the fragment reads are contiguous.
+// No barrier before the final sum, and LDS use does not depend on the row length.
+// Long rows of matrices with few tiles are cut in slices over workgroups (fp32
+// partial sums, added in slice order by whichever workgroup of the column
+// finishes last).
 #include "device_util.h"
 #include "internal.h"
 
@@ -65,10 +66,9 @@ struct StreamParams {
     uint32_t M, K, T;
     uint32_t rows;         // M, or 2*M when fp32 activations are carried as (value, remainder) pairs
     // The T steps are cut in `slices` runs of slice_steps (workgroups with blockIdx.y == s
-    // take run s); a workgroup walks its run in chunks of chunk_steps, the activations of
-    // one chunk in LDS at a time.  With more than one slice the workgroups write fp32
+    // take run s).  With more than one slice the workgroups write fp32
     // partial sums [slice][M][n_total] for the reduction kernel.
-    uint32_t slices, slice_steps, chunk_steps;
+    uint32_t slices, slice_steps;
     float *partials;
     // Non-null: the workgroups of one column (blockIdx.x) count their arrivals here after
     // writing their partial sums, and the one that arrives last adds all slices (in slice
@@ -113,12 +113,12 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     // issues its first weight loads a microsecond earlier.
     const uint32_t columns = p.columns, targets = p.targets, first1 = p.first_block[1],
                    first2 = p.first_block[2], first3 = p.first_block[3];
-    const uint32_t T = p.T, K = p.K, slice_steps = p.slice_steps, chunk_steps = p.chunk_steps, rows = p.rows;
+    const uint32_t T = p.T, K = p.K, slice_steps = p.slice_steps, rows = p.rows;
     const int fuse_silu = p.fuse_silu;
     const uint32_t *const ids = p.ids;
     const _Float16 *const x = p.x;
     asm volatile("" ::"s"(columns), "s"(targets), "s"(first1), "s"(first2), "s"(first3), "s"(T), "s"(K),
-                 "s"(slice_steps), "s"(chunk_steps), "s"(rows), "s"(fuse_silu), "s"(ids), "s"(x));
+                 "s"(slice_steps), "s"(rows), "s"(fuse_silu), "s"(ids), "s"(x));
     if (blockIdx.x >= columns) return;  // the grid is padded to a multiple of the XCD count
     uint32_t target = 0;
     if (1u < targets && blockIdx.x >= first1) target = 1;
@@ -547,7 +547,7 @@ q4_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__restric
 
 struct StreamShape {
     int mp, tb, depth, waves;
-    uint32_t slices, slice_steps, chunk_steps;
+    uint32_t slices, slice_steps;
 };
 
 // every wave's ring of activation slots (one more than its steps in flight from four rows on;
@@ -600,16 +600,12 @@ static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const
     }
 }
 
-// Cuts the T steps into slices (across workgroups) and each slice into chunks
-// (walked by one workgroup) whose activations take at most 40 KiB of LDS.
+// Cuts the T steps into slices (runs of steps taken by different workgroups).
 static void choose_cuts(StreamShape &shape, uint32_t T, uint32_t slices)
 {
-    const uint32_t max_steps = T;  // the activations pass through per-wave slots: no chunks
     slices = slices < 1u ? 1u : slices > T ? T : slices;
     shape.slice_steps = (T + slices - 1) / slices;
     shape.slices = (T + shape.slice_steps - 1) / shape.slice_steps;
-    const uint32_t chunks = (shape.slice_steps + max_steps - 1) / max_steps;
-    shape.chunk_steps = (shape.slice_steps + chunks - 1) / chunks;
 }
 
 static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp)
@@ -662,7 +658,7 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         if (fields >= 4 && fs >= 1) slices = (uint32_t)fs;
     }
     choose_cuts(shape, T, slices);
-    while (shape.waves > 2 && (uint32_t)shape.waves > shape.chunk_steps) shape.waves /= 2;
+    while (shape.waves > 2 && (uint32_t)shape.waves > shape.slice_steps) shape.waves /= 2;
     while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
         shape.waves /= 2;
     return shape;
@@ -731,7 +727,6 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.K = first.K;
     p.T = first.T;
     p.rows = rows;
-    p.chunk_steps = shape.chunk_steps;
     p.slice_steps = shape.slice_steps;
     p.slices = shape.slices;
     if (p.slices > 1u) {
@@ -762,9 +757,9 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     static const bool trace = getenv("MI355Q_TRACE") != nullptr;
     if (trace)
         fprintf(stderr, "mi355q: q4 stream rows=%u tiles=%u steps=%u -> %d tiles x %d waves per workgroup, "
-                        "depth %d, %u slices of %u steps in chunks of %u\n", rows, tiles, first.T, shape.tb,
+                        "depth %d, %u slices of %u steps\n", rows, tiles, first.T, shape.tb,
                 shape.waves, shape.depth, shape.slices,
-                shape.slice_steps, shape.chunk_steps);
+                shape.slice_steps);
     hipError_t launched;
     switch (mp) {
     case 1: launched = launch_shape<1>(ctx, p, shape); break;
