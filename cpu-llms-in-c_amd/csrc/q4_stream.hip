@@ -588,6 +588,9 @@ static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const
     case 10202: return launch_one<MP, 1, 2, 2>(ctx, p);
     case 10204: return launch_one<MP, 1, 2, 4>(ctx, p);
     case 10208: return launch_one<MP, 1, 2, 8>(ctx, p);
+    case 10216:
+        if constexpr (MP <= 2) return launch_one<MP, 1, 2, 16>(ctx, p);
+        return hipErrorInvalidValue;
     case 10404: return launch_one<MP, 1, 4, 4>(ctx, p);
     case 10408: return launch_one<MP, 1, 4, 8>(ctx, p);
     case 20202: return launch_one<MP, 2, 2, 2>(ctx, p);
@@ -620,12 +623,16 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         // One or two activation rows: a step's activations are a quarter or half of a 64-lane
         // load, so nothing is gained by sharing them between tiles; one tile per workgroup and
         // many workgroups stream best (gate|up at M = 1: 2176 workgroups of four waves 19.3 us,
-        // 1088 pairs of tiles 20.2-20.5; at M = 2 20.1 against 23.4), eight waves when the
-        // tiles are few (q|k|v 7.3 against 8.15 us with four).  Only a matrix with tens of
+        // 1088 pairs of tiles 20.2-20.5; at M = 2 20.1 against 23.4), eight waves or more when
+        // the tiles are few (q|k|v 7.3 against 8.15 us with four).  Only a matrix with tens of
         // thousands of tiles (the LM head) takes two or four per workgroup, two waves each.
         shape.tb = NT_total >= 32u * cus ? 4 : NT_total >= 12u * cus ? 2 : 1;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
         shape.waves = shape.tb > 1 ? 2 : groups <= 3u * cus ? 8 : 4;
+        // one row and two workgroups per compute unit (q|k|v: 512 tiles of 40 steps): sixteen
+        // waves put nearly the whole matrix in flight at once, 6.8-6.9 against 7.2-7.4 us
+        // (with two rows, or 320 tiles, eight are better)
+        if (mp == 1 && shape.tb == 1 && groups > cus + cus / 2u && groups <= 3u * cus) shape.waves = 16;
         if (NT_total <= cus + cus / 2u && T >= 96u) {
             // few tiles with long rows (the 27B down projection): K slices keep more loads in
             // flight than eight waves on a whole row.  With more tiles than compute units,
