@@ -49,7 +49,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X datasheet: 8 TB/s HBM3E
 # HBM bytes moved per algorithmic byte by the streaming kernel on the default workload: FETCH_SIZE and
 # WRITE_SIZE of rocprofv3 --pmc, scaled by a plain 2 GiB read/fill in the same runs
 # (profiles/q4_stream_kernel_layer_m1.md); a counter reading, not something this script can measure
-MEASURED_TRAFFIC_RATIO_LAYER_M1 = 1.007
+MEASURED_TRAFFIC_RATIO_LAYER_M1 = 1.006
 F16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 matrix instructions
 I8_MFMA_PEAK_TOPS = 5000.0  # dense int8 matrix instructions
 
