@@ -81,6 +81,15 @@ def test_fp32_activations(engine, oracle, gpu, M):
              engine.META_F16_INTERLEAVED, engine.F32, engine.F32, residual=True)
 
 
+@pytest.mark.parametrize("M", [2, 6])
+def test_fp32_activations_long_rows(engine, oracle, gpu, M):
+    """fp32 x on long rows with few tiles: the rows are cut in K slices that different workgroups
+    take (M = 6 runs as twelve fp16 rows, the widest activation slots), and K = 17472 is an odd
+    multiple of 64, so the last step has only its lower half."""
+    run_case(engine, oracle, gpu, 528, 17472, M, engine.META_BF16_PLANES, engine.F32, engine.F32,
+             seed=23, residual=True)
+
+
 @pytest.mark.parametrize("y_dtype", ["F16", "BF16", "F32"])
 def test_bf16_activations_and_outputs(engine, oracle, gpu, y_dtype):
     """bf16 activations and outputs (minimax_h3_m3_run_q4_projection_bf16)."""
