@@ -433,6 +433,11 @@ def main():
     # kernel time of each step (its launches, and the slice reductions some of them carry)
     per_step = per_launch[:len(per_launch) // args.steps * args.steps].reshape(args.steps, -1).sum(axis=1)
     p10, p50, p90 = (float(np.percentile(per_step, q)) for q in (10, 50, 90))
+    # median duration of each launch of a step, in launch order (only when every launch is one kernel)
+    launch_p50 = None
+    if len(per_launch) == args.steps * launches_per_step:
+        launch_p50 = [round(float(v), 2)
+                      for v in np.median(per_launch.reshape(args.steps, launches_per_step), axis=0)]
 
     # measured plain-read ceiling: whole 2 GiB pass, and launches the size of one weight matrix
     read_long = ctx.probe_read_bandwidth(2 << 30, 3, 1, 0)
@@ -475,6 +480,7 @@ def main():
             "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
             "kernel_us_per_step_p10_p50_p90": [round(p10, 2), round(p50, 2), round(p90, 2)],
             "gb_per_s_at_p50_kernel_time": round(step_bytes / (p50 * 1e-6) / 1e9, 1),
+            "kernel_us_per_launch_p50_in_launch_order": launch_p50,
             "weights_sha256": weights_digest(host, shapes),
             "device": info.name.decode(errors="replace").strip(),
             "arch": info.arch.decode(errors="replace"),
