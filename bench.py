@@ -185,7 +185,9 @@ def common_fields(args, wall):
 
 def device_fields(info):
     return {"device": info.name.decode(errors="replace").strip(),
-            "arch": info.arch.decode(errors="replace"), "compute_units": info.compute_units}
+            "arch": info.arch.decode(errors="replace"),
+            "max_clock_mhz": info.clock_mhz, "memory_clock_mhz": info.memory_clock_mhz,
+            "memory_bus_bits": info.memory_bus_bits, "compute_units": info.compute_units}
 
 
 def bench_prefill(engine, ctx, args):
@@ -484,6 +486,8 @@ def main():
             "weights_sha256": weights_digest(host, shapes),
             "device": info.name.decode(errors="replace").strip(),
             "arch": info.arch.decode(errors="replace"),
+            "max_clock_mhz": info.clock_mhz, "memory_clock_mhz": info.memory_clock_mhz,
+            "memory_bus_bits": info.memory_bus_bits,
             "compute_units": info.compute_units,
             "measured_read_gb_per_s": {"one_2GiB_pass": round(read_long, 1),
                                        "matrix_sized_launches": round(read_short, 1)},
