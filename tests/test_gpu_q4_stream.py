@@ -112,6 +112,29 @@ def test_repeat_calls_are_bitwise_stable(engine, gpu):
         weight.destroy()
 
 
+def test_back_to_back_launches_of_mixed_row_counts(engine, oracle, gpu):
+    """Launches with different numbers of activation rows lay LDS out differently (a wave's
+    activation slots grow with the rows).  Many of them back to back on one weight, the workgroups
+    of one launch taking over the LDS of the previous one's: every result equals the first of its
+    kind bit for bit, and the first of each kind passes the usual gate."""
+    N, K = 1536, 2112  # K: an odd multiple of 64
+    quants, meta_a, meta_b = engine.synth_q4_affine(31, 0.02, N, K, engine.META_BF16_PLANES)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+    try:
+        inputs = {M: make_x(engine, 40 + M, M, K, engine.F16) for M in (1, 2, 5, 8, 16)}
+        first = {}
+        for M, x in inputs.items():
+            first[M] = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+            ref = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x, engine.F16, M)
+            assert q4_relative_error(first[M], ref) <= TOLERANCE
+        for _ in range(20):
+            for M in (16, 1, 8, 2, 5):
+                again = gpu.q4_linear(weight, inputs[M], engine.F16, engine.F32)
+                assert np.array_equal(first[M].view(np.uint32), again.view(np.uint32)), f"M={M}"
+    finally:
+        weight.destroy()
+
+
 def test_argument_errors(engine, gpu):
     quants, meta_a, meta_b = engine.synth_q4_affine(1, 0.02, 16, 64, engine.META_F16_INTERLEAVED)
     with pytest.raises(engine.Mi355qError) as info:
