@@ -47,7 +47,51 @@ int ensure_stage(mi355q_context *ctx, int slot, size_t bytes, char *error,
 
 using namespace mi355q;
 
+// One experiment knob of a context; an empty or null value clears it.
+static int apply_option(mi355q_context *ctx, const char *name, const char *value)
+{
+    const bool set = value != nullptr && value[0] != '\0';
+    if (strcmp(name, "q4_stream") == 0) {  // "TILES,DEPTH,WAVES[,SLICES]"
+        int f[4] = {0, 0, 0, 0};
+        if (set && sscanf(value, "%d,%d,%d,%d", &f[0], &f[1], &f[2], &f[3]) < 3) return MI355Q_ERROR_INVALID;
+        if (set && (f[0] < 1 || f[1] < 1 || f[2] < 1 || f[3] < 0)) return MI355Q_ERROR_INVALID;
+        memcpy(ctx->force_stream, f, sizeof f);
+        return MI355Q_OK;
+    }
+    if (strcmp(name, "q4_gemm") == 0) {  // "VARIANT,SPLITS"
+        int f[2] = {0, 0};
+        if (set && (sscanf(value, "%d,%d", &f[0], &f[1]) != 2 || f[0] < 0 || f[1] < 1 || f[1] > 16))
+            return MI355Q_ERROR_INVALID;
+        memcpy(ctx->force_gemm, f, sizeof f);
+        return MI355Q_OK;
+    }
+    if (strcmp(name, "trace") == 0) {
+        ctx->trace = set && strcmp(value, "0") != 0;
+        return MI355Q_OK;
+    }
+    if (strcmp(name, "in_kernel_slices") == 0) {  // "0": a second kernel adds the K slices
+        ctx->columns_share_xcd = ctx->columns_probed && !(set && strcmp(value, "0") == 0);
+        return MI355Q_OK;
+    }
+    return MI355Q_ERROR_INVALID;
+}
+
 extern "C" {
+
+int mi355q_context_set_option(mi355q_context *ctx, const char *name, const char *value, char *error,
+                              size_t error_capacity)
+{
+    if (ctx == nullptr || name == nullptr) {
+        set_error(error, error_capacity, "context_set_option: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (apply_option(ctx, name, value) != MI355Q_OK) {
+        set_error(error, error_capacity, "context_set_option: unknown option or malformed value: %s=%s", name,
+                  value ? value : "");
+        return MI355Q_ERROR_INVALID;
+    }
+    return MI355Q_OK;
+}
 
 int mi355q_context_create(int device, mi355q_context **out, char *error,
                           size_t error_capacity)
@@ -87,7 +131,12 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipMemset(ctx->arrivals, 0, kArrivalCounters * sizeof(uint32_t));
     uint32_t xcds = 0;
     if (status == hipSuccess) status = probe_columns_share_xcd(ctx, &ctx->columns_share_xcd, &xcds);
-    if (getenv("MI355Q_NO_ARRIVALS") != nullptr) ctx->columns_share_xcd = false;  // for comparisons
+    ctx->columns_probed = ctx->columns_share_xcd;
+    // the environment is read here, once per context, and nowhere on the call path
+    if (getenv("MI355Q_NO_ARRIVALS") != nullptr) (void)apply_option(ctx, "in_kernel_slices", "0");
+    (void)apply_option(ctx, "q4_stream", getenv("MI355Q_Q4_STREAM"));
+    (void)apply_option(ctx, "q4_gemm", getenv("MI355Q_Q4_GEMM"));
+    (void)apply_option(ctx, "trace", getenv("MI355Q_TRACE"));
     if (status != hipSuccess) {
         int code = fail_hip(status, "context_create", error, error_capacity);
         mi355q_context_destroy(ctx);

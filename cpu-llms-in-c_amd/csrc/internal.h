@@ -69,6 +69,14 @@ struct mi355q_context {
     // the workgroup that arrives last adds the slices and puts its counter back to zero
     uint32_t *arrivals;
     bool columns_share_xcd;  // probed at creation; false switches that addition to a second kernel
+    bool columns_probed;     // what the probe said (columns_share_xcd can be switched off by an option)
+    // Experiment knobs, read from the environment once at creation (MI355Q_Q4_STREAM,
+    // MI355Q_Q4_GEMM, MI355Q_TRACE, MI355Q_NO_ARRIVALS) and settable per context with
+    // mi355q_context_set_option; nothing on the call path reads the environment.
+    int force_stream[4];  // tiles, depth, waves, slices (0 = not forced); [0] == 0: no forcing
+    int force_gemm[2];    // kernel variant, K splits; [1] == 0: no forcing
+    bool trace;           // print the chosen decomposition of every launch to stderr
+    bool lds_raised[16];  // q4_gemm_pipe_kernel instantiations whose dynamic LDS limit has been raised
 };
 namespace mi355q {
 constexpr uint32_t kArrivalCounters = 65536;

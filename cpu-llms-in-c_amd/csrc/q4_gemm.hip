@@ -455,10 +455,15 @@ __device__ __forceinline__ void touch(T &a, T &b, T &c, T &d)
 template <int IMMEDIATE>
 __device__ __forceinline__ void load_to_lds(uint32_t lane_offset, const char *base, uint32_t lds_base)
 {
+    // m0 is named as clobbered so that the compiler carries no value of its own in it across
+    // the statement (it warns that m0 is reserved, which is the point)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
     asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2"
                  :
                  : "v"(lane_offset), "s"(base), "n"(IMMEDIATE), "s"(lds_base)
-                 : "memory");
+                 : "memory", "m0");
+#pragma clang diagnostic pop
 }
 __device__ __forceinline__ void load_x4(u32x4 &to, uint32_t lane_offset, const char *base)
 {
@@ -789,7 +794,8 @@ q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__re
 {
     const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (index >= count) return;
-    out[index] = (_Float16)load_as_float(x, x_dtype, index);
+    const float value = load_as_float(x, x_dtype, index), limit = 65504.0f;  // saturate, no infinities
+    out[index] = (_Float16)(value > limit ? limit : value < -limit ? -limit : value);
 }
 
 // The pipelined kernel's stage is larger than the 64 KiB a kernel gets without asking: the
@@ -797,15 +803,16 @@ q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__re
 template <int NTW, bool XT>
 static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &p)
 {
-    static bool raised[64] = {};
     constexpr size_t bytes = pipe_lds_bytes(128);
-    const int device = ctx->device;
-    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    if (!raised[device]) {
+    constexpr int slot = 2 * NTW + (XT ? 1 : 0);  // this instantiation's flag in the context
+    static_assert(slot < 16, "mi355q_context::lds_raised holds sixteen flags");
+    // per context (a context belongs to one device and serialises its calls): no process-wide
+    // state, so contexts on different threads do not meet here; raising the limit twice is harmless
+    if (!ctx->lds_raised[slot]) {
         hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, NTW, XT>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (status != hipSuccess) return status;
-        raised[device] = true;
+        ctx->lds_raised[slot] = true;
     }
     return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT>, grid, dim3(256), bytes, p);
 }
@@ -920,15 +927,13 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             }
         }
     }
-    const char *force = getenv("MI355Q_Q4_GEMM");  // "VARIANT,SPLITS" for experiments
-    int fv = 0, fs = 0;
-    if (force && sscanf(force, "%d,%d", &fv, &fs) == 2 && fv >= 0 &&
-        fv < (int)(sizeof variants / sizeof variants[0]) && fs >= 1 && fs <= 16 && (fv < 6 || pipe_ok)) {
-        best = fv;
-        best_splits = (uint32_t)fs;
+    // option "q4_gemm" = "VARIANT,SPLITS" for experiments
+    if (ctx->force_gemm[1] >= 1 && ctx->force_gemm[0] < (int)(sizeof variants / sizeof variants[0]) &&
+        (ctx->force_gemm[0] < 6 || pipe_ok)) {
+        best = ctx->force_gemm[0];
+        best_splits = (uint32_t)ctx->force_gemm[1];
     }
-    static const bool trace = getenv("MI355Q_TRACE") != nullptr;
-    if (trace)
+    if (ctx->trace)
         fprintf(stderr, "mi355q: q4 gemm M=%u N=%u K=%u -> variant %d (BM=%d, %d tiles/wave%s), K split %u\n",
                 a.M, w.N, w.K, best, variants[best].bm, variants[best].ntw,
                 variants[best].extra ? " +1" : "", best_splits);

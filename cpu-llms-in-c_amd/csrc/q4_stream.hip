@@ -35,6 +35,8 @@
 
 namespace mi355q {
 
+constexpr size_t kRowScaleBytes = 256;  // one float per activation row in front of converted rows
+
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
 // compile-time constant in the body
 template <int... I, class F>
@@ -63,6 +65,10 @@ struct StreamParams {
     uint32_t matrix_rows;
     uint32_t targets;
     const _Float16 *x;  // [rows][K] fp16
+    // Activations that were converted to fp16 were first scaled, row by row, by a power of two
+    // that brings the row's largest magnitude to [2^13, 2^14); row_scale[m] is the inverse power,
+    // by which the finished dot products of row m are multiplied.  Null: fp16 activations as given.
+    const float *row_scale;
     uint32_t M, K, T;
     uint32_t rows;         // M, or 2*M when fp32 activations are carried as (value, remainder) pairs
     // The T steps are cut in `slices` runs of slice_steps (workgroups with blockIdx.y == s
@@ -227,10 +233,15 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 const uint32_t offset = tail_step ? x_lane_tail[b] : x_lane[b];
                 // the slot was last read by the step consumed before this fetch: those LDS reads
                 // have returned before the write can land (wait for them all the same)
+                // (m0 is named as clobbered so that the compiler does not carry a value of its
+                // own in it across the statement; it warns that m0 is reserved, which is the point)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                              :
                              : "v"(offset), "s"(x_at), "s"(lds_wave + slot_bytes + 1024u * (uint32_t)b)
-                             : "memory");
+                             : "memory", "m0");
+#pragma clang diagnostic pop
             }
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb) {
@@ -427,6 +438,11 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 continue;
             }
             const size_t at = (size_t)m * N + n;
+            if (p.row_scale) {
+                const float back = p.row_scale[m];
+                value *= back;
+                value_up *= back;
+            }
             if (fuse_here) {
                 store_from_float(p.y[0], p.y_dtype, at, silu_times(value, value_up));
                 continue;
@@ -445,10 +461,13 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     // The workgroups of one column run on the same XCD (the grid's width is a multiple of the
     // number of XCDs, over which workgroups are dealt round-robin in launch order), so they
     // share one L2: the partial sums and the counter are written and read there (agent-scope
-    // accesses, which pass the per-CU cache), and a thread only has to know its stores have
-    // been acknowledged before the count goes up.  No device-wide cache write-back.
+    // accesses, which pass the per-CU cache).  The count may go up only after every thread's
+    // partial sums have been acknowledged by L2: each thread waits for its own stores
+    // (vmcnt counts stores on this target; a workgroup-scope fence alone emits no such wait),
+    // then the barrier joins the threads, then thread 0 counts.  No device-wide cache write-back.
     __shared__ uint32_t last_arrival;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this thread's stores have reached L2
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this thread's stores have reached L2
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // and the compiler moves nothing across
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t before =
@@ -478,10 +497,11 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
             }
             return sum;
         };
-        float value = total(p.n_first[slot_target] + n);
+        const float back = p.row_scale ? p.row_scale[m] : 1.0f;
+        float value = total(p.n_first[slot_target] + n) * back;
         const size_t at = (size_t)m * N + n;
         if (p.fuse_silu) {
-            store_from_float(p.y[0], p.y_dtype, at, silu_times(value, total(p.n_first[1] + n)));
+            store_from_float(p.y[0], p.y_dtype, at, silu_times(value, total(p.n_first[1] + n) * back));
             continue;
         }
         if (p.residual[target])
@@ -505,6 +525,8 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
     float value = 0.0f;
     for (uint32_t s = 0; s < p.slices; ++s)
         value += p.partials[((size_t)s * p.M + m) * p.n_total + column];
+    const float back = p.row_scale ? p.row_scale[m] : 1.0f;
+    value *= back;
     const uint32_t n = column - p.n_first[target];
     const size_t at = (size_t)m * p.N[target] + n;
     if (p.fuse_silu) {  // columns [0, N) hold gate . x, [N, 2N) hold up . x
@@ -512,7 +534,7 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
         float value_up = 0.0f;
         for (uint32_t s = 0; s < p.slices; ++s)
             value_up += p.partials[((size_t)s * p.M + m) * p.n_total + p.n_first[1] + n];
-        store_from_float(p.y[0], p.y_dtype, at, silu_times(value, value_up));
+        store_from_float(p.y[0], p.y_dtype, at, silu_times(value, value_up * back));
         return;
     }
     if (p.residual[target])
@@ -521,25 +543,54 @@ __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParam
     store_from_float(p.y[target], p.y_dtype, at, value);
 }
 
-// Activations that are not fp16 are converted once per call into fp16 rows:
-// bf16 -> fp16 (exact inside fp16's normal range), fp32 -> two rows per input
-// row: the value rounded to fp16 and the rounding remainder, whose results the
-// kernel adds (about 22 significant bits of x survive).
-__global__ void __launch_bounds__(256)
+// Activations that are not fp16 are converted once per call into fp16 rows, one workgroup
+// per input row.  The row is first scaled by the power of two that brings its largest finite
+// magnitude into [2^13, 2^14) (exact in fp32), so that fp16's narrow exponent range costs
+// nothing whatever the row's own magnitude is; row_scale[m] receives the inverse power, which
+// the kernel's epilogue multiplies back in.  bf16 -> one fp16 row (exact down to 2^-27 of the
+// row's maximum); fp32 -> two rows: the value rounded to fp16 and the rounding remainder,
+// whose results the kernel adds (about 22 significant bits relative to the row's maximum).
+// Infinities saturate at the largest fp16 value, NaN stays NaN.
+constexpr uint32_t kConvertThreads = 1024;
+__global__ void __launch_bounds__(kConvertThreads)
 q4_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__restrict__ out,
-                    uint32_t M, uint32_t K)
+                    float *__restrict__ row_scale, uint32_t M, uint32_t K)
 {
-    const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (index >= (size_t)M * K) return;
-    const uint32_t m = (uint32_t)(index / K), k = (uint32_t)(index % K);
-    if (x_dtype == MI355Q_BF16) {
-        uint32_t bits = ((const uint16_t *)x)[index];
-        out[index] = (_Float16)__builtin_bit_cast(float, bits << 16);
-    } else {
-        float value = ((const float *)x)[index];
-        _Float16 head = (_Float16)value;
-        out[(size_t)(2u * m) * K + k] = head;
-        out[(size_t)(2u * m + 1u) * K + k] = (_Float16)(value - (float)head);
+    __shared__ float wave_max[kConvertThreads / 64u];
+    const uint32_t m = blockIdx.x;
+    const size_t row_at = (size_t)m * K;
+    float biggest = 0.0f;
+    for (uint32_t k = threadIdx.x; k < K; k += kConvertThreads) {
+        const float magnitude = __builtin_fabsf(load_as_float(x, x_dtype, row_at + k));
+        if (magnitude > biggest && magnitude <= 3.4028234e38f) biggest = magnitude;  // finite values only
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        const float other = __shfl_xor(biggest, offset, 64);
+        biggest = other > biggest ? other : biggest;
+    }
+    if ((threadIdx.x & 63u) == 0u) wave_max[threadIdx.x >> 6] = biggest;
+    __syncthreads();
+    biggest = wave_max[0];
+#pragma unroll
+    for (uint32_t w = 1; w < kConvertThreads / 64u; ++w) biggest = wave_max[w] > biggest ? wave_max[w] : biggest;
+    int exponent = 0;
+    (void)__builtin_frexpf(biggest, &exponent);  // biggest = f * 2^exponent, f in [0.5, 1)
+    int shift = biggest > 0.0f ? 14 - exponent : 0;
+    shift = shift < -126 ? -126 : shift > 126 ? 126 : shift;  // both powers stay normal numbers
+    const float forward = __builtin_ldexpf(1.0f, shift), back = __builtin_ldexpf(1.0f, -shift);
+    if (threadIdx.x == 0) row_scale[m] = back;
+    const float limit = 65504.0f;
+    for (uint32_t k = threadIdx.x; k < K; k += kConvertThreads) {
+        const float value = load_as_float(x, x_dtype, row_at + k) * forward;
+        const _Float16 head = (_Float16)(value > limit ? limit : value < -limit ? -limit : value);
+        if (x_dtype == MI355Q_BF16) {
+            out[row_at + k] = head;
+        } else {
+            const float rest = value - (float)head;
+            out[(size_t)(2u * m) * K + k] = head;
+            out[(size_t)(2u * m + 1u) * K + k] = (_Float16)(rest > limit ? limit : rest < -limit ? -limit : rest);
+        }
     }
 }
 
@@ -654,15 +705,11 @@ static StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, ui
         const uint32_t want = 16u * cus / (groups * shape.slices);
         shape.waves = want <= 2u ? 2 : want < 8u ? 4 : 8;
     }
-    // "TB,DEPTH,WAVES[,SLICES]" for experiments
-    const char *force = getenv("MI355Q_Q4_STREAM");
-    int ft = 0, fd = 0, fw = 0, fs = 0;
-    const int fields = force ? sscanf(force, "%d,%d,%d,%d", &ft, &fd, &fw, &fs) : 0;
-    if (fields >= 3) {
-        shape.tb = ft;
-        shape.depth = fd;
-        shape.waves = fw;
-        if (fields >= 4 && fs >= 1) slices = (uint32_t)fs;
+    if (ctx->force_stream[0] > 0) {  // option "q4_stream" = "TILES,DEPTH,WAVES[,SLICES]" for experiments
+        shape.tb = ctx->force_stream[0];
+        shape.depth = ctx->force_stream[1];
+        shape.waves = ctx->force_stream[2];
+        if (ctx->force_stream[3] >= 1) slices = (uint32_t)ctx->force_stream[3];
     }
     choose_cuts(shape, T, slices);
     while (shape.waves > 2 && (uint32_t)shape.waves > shape.slice_steps) shape.waves /= 2;
@@ -687,16 +734,19 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     memset(&p, 0, sizeof p);
     p.x = (const _Float16 *)a.x;
     if (a.x_dtype != MI355Q_F16) {
-        const size_t bytes = (size_t)rows * first.K * sizeof(_Float16);
+        // [ the rows' inverse scales (16 floats, 256 bytes) | rows * K fp16 ]
+        const size_t bytes = kRowScaleBytes + (size_t)rows * first.K * sizeof(_Float16);
         int status = ensure_stage(ctx, 3, bytes, error, error_capacity);
         if (status != MI355Q_OK) return status;
-        const size_t count = (size_t)a.M * first.K;
-        hipError_t converted =
-            launch(ctx, q4_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256), 0,
-                   a.x, a.x_dtype, (_Float16 *)ctx->stage[3], a.M, first.K);
+        unsigned char *const area = (unsigned char *)ctx->stage[3];
+        float *const row_scale = (float *)area;
+        _Float16 *const converted_x = (_Float16 *)(area + kRowScaleBytes);
+        hipError_t converted = launch(ctx, q4_convert_x_kernel, dim3(a.M), dim3(kConvertThreads), 0, a.x,
+                                      a.x_dtype, converted_x, row_scale, a.M, first.K);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
-        p.x = (const _Float16 *)ctx->stage[3];
+        p.x = converted_x;
+        p.row_scale = row_scale;
     }
     const bool subset = a.row_count != 0u;
     if (subset && (a.count != 1u || a.fuse_silu || a.targets[0].residual != nullptr ||
@@ -710,6 +760,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         tiles += subset ? (a.row_count + kTileRows - 1) / kTileRows : a.targets[t].w->NT;
     StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
     if (a.fuse_silu && shape.tb != 2 && shape.tb != 4) shape.tb = 2;  // gate and up tiles pair up
+    if (shape.tb > 1 && shape.waves > 8) shape.waves = 8;  // sixteen waves exist for single tiles only
     while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
         shape.waves /= 2;
     uint32_t block = 0;
@@ -741,12 +792,12 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
             p.n_first[t] = p.n_total;
             p.n_total += p.N[t];
         }
-        int status = ensure_stage(ctx, 4, (size_t)p.slices * a.M * p.n_total * sizeof(float), error,
-                                  error_capacity);
-        if (status != MI355Q_OK) return status;
-        p.partials = (float *)ctx->stage[4];
+        const size_t partial_bytes = (size_t)p.slices * a.M * p.n_total * sizeof(float);
         // grid.x of the launch: the workgroup columns that count arrivals
         const uint32_t columns = a.fuse_silu ? (p.NT[0] + shape.tb / 2 - 1) / (shape.tb / 2) : block;
+        int status = ensure_stage(ctx, 4, partial_bytes, error, error_capacity);
+        if (status != MI355Q_OK) return status;
+        p.partials = (float *)ctx->stage[4];
         p.arrivals = ctx->columns_share_xcd && columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
     }
     p.pair = pair;
@@ -761,8 +812,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
                   lds, first.K, rows);
         return MI355Q_ERROR_INVALID;
     }
-    static const bool trace = getenv("MI355Q_TRACE") != nullptr;
-    if (trace)
+    if (ctx->trace)
         fprintf(stderr, "mi355q: q4 stream rows=%u tiles=%u steps=%u -> %d tiles x %d waves per workgroup, "
                         "depth %d, %u slices of %u steps\n", rows, tiles, first.T, shape.tb,
                 shape.waves, shape.depth, shape.slices,
@@ -774,6 +824,12 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     case 4: launched = launch_shape<4>(ctx, p, shape); break;
     case 8: launched = launch_shape<8>(ctx, p, shape); break;
     default: launched = launch_shape<16>(ctx, p, shape); break;
+    }
+    if (launched == hipErrorInvalidValue) {  // no such instantiation (the launch itself reports other codes)
+        set_error(error, error_capacity, "q4 stream kernel: no kernel for %d rows, %d tiles, depth %d, %d waves",
+                  mp, shape.tb, shape.depth, shape.waves);
+        (void)hipGetLastError();
+        return MI355Q_ERROR_INVALID;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 stream kernel launch", error, error_capacity);

@@ -63,6 +63,7 @@ SIGNATURES = {
     "mi355q_context_create": (_int, [_int, _c.POINTER(_vp), *_err]),
     "mi355q_context_destroy": (None, [_vp]),
     "mi355q_context_info": (_int, [_vp, _c.POINTER(DeviceInfo), *_err]),
+    "mi355q_context_set_option": (_int, [_vp, _cp, _cp, *_err]),
     "mi355q_sync": (_int, [_vp, *_err]),
     "mi355q_device_alloc": (_int, [_vp, _sz, _c.POINTER(_vp), *_err]),
     "mi355q_device_free": (_int, [_vp, _vp, *_err]),
@@ -244,6 +245,11 @@ class Context:
         info = DeviceInfo()
         _call(self.lib.mi355q_context_info, self.handle, ctypes.byref(info))
         return info
+
+    def set_option(self, name: str, value: str | None):
+        """Experiment knob of this context (see mi355q_context_set_option); None clears it."""
+        _call(self.lib.mi355q_context_set_option, self.handle, name.encode(),
+              None if value is None else value.encode())
 
     def sync(self):
         _call(self.lib.mi355q_sync, self.handle)

@@ -113,6 +113,18 @@ int mi355q_context_create(int device, mi355q_context **out,
 void mi355q_context_destroy(mi355q_context *ctx);
 int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
                         char *error, size_t error_capacity);
+/* Experiment knobs of one context — the counterpart of the reference's QWEN38_* /
+ * MINIMAX_* environment switches that its benches read (qwen38_m3_decode.m:1217-1283
+ * QWEN38_PROFILE; qwen38_m3.m:342-345).  The environment variables MI355Q_Q4_STREAM,
+ * MI355Q_Q4_GEMM, MI355Q_TRACE and MI355Q_NO_ARRIVALS are read once, when the context is
+ * created; this call changes the same knobs afterwards.  A NULL or empty value clears one.
+ *   "q4_stream" = "TILES,DEPTH,WAVES[,SLICES]"  forces the streaming kernel's launch shape
+ *   "q4_gemm"   = "VARIANT,SPLITS"              forces the GEMM's kernel variant and K split
+ *   "trace"     = "1"                           prints every launch's decomposition to stderr
+ *   "in_kernel_slices" = "0"                    K slices are added by a second kernel
+ * Unknown names and malformed values: status 2. */
+int mi355q_context_set_option(mi355q_context *ctx, const char *name, const char *value,
+                              char *error, size_t error_capacity);
 /* Waits for everything queued on the context's stream
  * (the reference's waitUntilCompleted, qwen38_m3_decode.m:1701-1716). */
 int mi355q_sync(mi355q_context *ctx, char *error, size_t error_capacity);

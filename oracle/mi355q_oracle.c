@@ -535,7 +535,8 @@ void orc_w8a8_conv(const uint8_t *weights, uint32_t N, uint32_t K, const int8_t 
  * Follows compiler/compile_minimindo_sensevoice_image.py:38-46 (q8_payload):
  * scale = max|w|/127 in double (1.0 for an all-zero row), stored as fp32;
  * q = clamp(round_half_even(w / scale), -127, 127) with the division done in
- * fp32 against the fp32-rounded scale.  PARITY UNPINNED (see header). */
+ * fp32 against the fp32-rounded scale.  Pinned byte for byte by the records the
+ * reference function itself wrote for seeded inputs (tests/golden/q8_payload.npz). */
 void orc_q8_weight_quantize(const float *w, uint32_t N, uint32_t K, uint8_t *rows_out)
 {
     for (uint32_t n = 0; n < N; ++n) {
@@ -557,3 +558,32 @@ void orc_q8_weight_quantize(const float *w, uint32_t N, uint32_t K, uint8_t *row
         }
     }
 }
+
+/* The reference's synthetic affine-Q4 matrix of its Qwen3.8 benchmark (fill_weights,
+ * qwen38_m3.m:64-87): xorshift32 (<<13, >>17, <<5); per 64-column group 32 code bytes
+ * = the low byte of successive draws, then scale = 0.0035 + 0.00025 * (draw & 7) and
+ * bias = -7.5 * scale + 0.0002 * ((group % 5) - 2) in fp32, both stored as fp16.
+ * Seeds: gate 0x36a110c, up 0x27b4c51, down 0x36d027b (qwen38_m3.m:573-580).
+ * meta_interleaved receives {scale, bias} pairs.  An input recipe, not arithmetic of
+ * the path; pinned by the numpy restatement of the same formulas on the first rows. */
+void orc_recipe_qwen38_weights(uint32_t seed, size_t group_count, uint8_t *quants,
+                               uint16_t *meta_interleaved)
+{
+    uint32_t state = seed;
+    for (size_t index = 0; index < group_count; ++index) {
+        for (size_t byte = 0; byte < 32; ++byte) {
+            state ^= state << 13;
+            state ^= state >> 17;
+            state ^= state << 5;
+            quants[index * 32 + byte] = (uint8_t)state;
+        }
+        state ^= state << 13;
+        state ^= state >> 17;
+        state ^= state << 5;
+        const float scale = 0.0035f + 0.00025f * (float)(state & 7u);
+        const float bias = -7.5f * scale + 0.0002f * (float)((int)(index % 5) - 2);
+        meta_interleaved[2 * index] = orc_f32_to_f16(scale);
+        meta_interleaved[2 * index + 1] = orc_f32_to_f16(bias);
+    }
+}
+

@@ -27,11 +27,14 @@
  *   orc_quantize_i8 / orc_w8a8_*      the reference's own compiled
  *                                     quantize_i8 / matrix_i8_rows
  *                                     (oracle/_ref) and integer brute force
- *   orc_q8_weight_quantize            PARITY UNPINNED: the reference function
- *                                     is Python+torch (q8_payload) and is not
- *                                     executed; only its clamp/tie behaviour is
- *                                     checked against numpy.  It is an offline
- *                                     packer; the GEMM consumes its bytes.
+ *   orc_q8_weight_quantize            the record bytes the reference's own
+ *                                     q8_payload wrote for seeded matrices
+ *                                     (tests/golden/q8_payload.npz: ordinary
+ *                                     rows, quotients on and beside every .5,
+ *                                     zero and constant rows, extreme ranges),
+ *                                     byte for byte; likely wrong variants
+ *                                     (reciprocal multiply, halves away from
+ *                                     zero, double division) fail on it
  */
 #ifndef MI355Q_ORACLE_H
 #define MI355Q_ORACLE_H
@@ -136,6 +139,11 @@ void orc_w8a8_conv(const uint8_t *weights, uint32_t N, uint32_t K, const int8_t 
                    const float *x_scales, uint32_t M, const float *bias, float *out);
 void orc_q8_weight_quantize(const float *w, uint32_t N, uint32_t K,
                             uint8_t *rows_out);
+
+/* Input recipe of the reference's Qwen3.8 benchmark (qwen38_m3.m:64-87): xorshift32 code
+ * bytes and fp16 {scale, bias} pairs for group_count groups. */
+void orc_recipe_qwen38_weights(uint32_t seed, size_t group_count, uint8_t *quants,
+                               uint16_t *meta_interleaved);
 
 #ifdef __cplusplus
 }

@@ -75,6 +75,8 @@ def lib() -> ctypes.CDLL:
         l.orc_w8a8_linear.argtypes = [_vp, _u32, _u32, _vp, _vp, _u32, _vp, _vp, _vp, _int]
         l.orc_q8_weight_quantize.restype = None
         l.orc_q8_weight_quantize.argtypes = [_vp, _u32, _u32, _vp]
+        l.orc_recipe_qwen38_weights.restype = None
+        l.orc_recipe_qwen38_weights.argtypes = [_u32, _sz, _vp, _vp]
         _libs["oracle"] = l
     return _libs["oracle"]
 

@@ -39,6 +39,21 @@ def gpu(engine):
     context.close()
 
 
+@pytest.fixture
+def force(gpu):
+    """force(name, value): sets an experiment knob of the shared context (launch shape, kernel
+    variant) for the duration of one test."""
+    names = []
+
+    def apply(name, value):
+        gpu.set_option(name, value)
+        names.append(name)
+
+    yield apply
+    for name in names:
+        gpu.set_option(name, None)
+
+
 def q4_relative_error(y, reference):
     """max_i |y_i - ref_i| / max(|ref_i|, 1e-2 * rms(ref)), per activation row."""
     y = np.asarray(y, dtype=np.float64)

@@ -66,7 +66,7 @@ def test_edge_shapes(engine, oracle, gpu, N, K, M):
 
 @pytest.mark.parametrize("name,N,K", [("q", 6144, 5120), ("kv", 1024, 5120), ("o", 5120, 6144),
                                       ("gate_up", 17408, 5120), ("down", 5120, 17408)])
-@pytest.mark.parametrize("M", [1, 4, 8])
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
 def test_27b_layer_shapes(engine, oracle, gpu, name, N, K, M):
     """Headline configurations 2 and 3 (27B layer shapes, decode and verify): bf16 scale/bias, fp16 activations, fp16 output."""
     run_case(engine, oracle, gpu, N, K, M, engine.META_BF16_PLANES, engine.F16, engine.F16,
@@ -189,12 +189,16 @@ def test_shared_activation_multi_launch(engine, oracle, gpu, M):
 
 @pytest.mark.parametrize("N,K,M,x_dtype", [(1000, 1536, 1, "F16"), (1000, 1536, 3, "F16"),
                                            (2048, 1024, 8, "BF16"), (640, 8704, 8, "F16"),
-                                           (640, 8704, 4, "F32"), (17408, 5120, 1, "F16")])
+                                           (640, 8704, 4, "F32"), (17408, 5120, 1, "F16"),
+                                           (4096, 4096, 1, "F16"), (5120, 2048, 1, "F16"),
+                                           (3200, 1024, 2, "F16")])
 def test_fused_gate_up_silu(engine, oracle, gpu, N, K, M, x_dtype):
     """MI355Q_FUSE_GATE_UP_SILU: y = silu(gate . x) * (up . x) in one launch
     (qwen38_q4_gate_up_silu, qwen38_q4.metal:129-151), against the oracle's two exact-weight dots
     combined in float64; (640, 8704) is cut in K slices, so the reduction kernel applies the
-    nonlinearity there.  Also through the sequence call, with device pointers."""
+    nonlinearity there; N = 3200 .. 5120 at one row is the range where the unfused launch would
+    take sixteen waves per tile, which the paired tiles of the fused launch do not have.  Also
+    through the sequence call, with device pointers."""
     x_dtype = getattr(engine, x_dtype)
     gate_image = engine.synth_q4_affine(21, 0.02, N, K, engine.META_BF16_PLANES)
     up_image = engine.synth_q4_affine(22, 0.02, N, K, engine.META_BF16_PLANES)
@@ -346,32 +350,107 @@ def test_row_subset_with_device_ids(engine, oracle, gpu):
     assert np.array_equal(y[:, good].view(np.uint32), host.view(np.uint32))
 
 
-def test_slices_added_in_kernel_match_second_kernel(engine, oracle, gpu, monkeypatch):
+def test_activation_range(engine, oracle, gpu):
+    """Activations far from fp16's range.  Rows that are not fp16 are scaled by a power of two
+    per row before they are split into fp16 pieces, so the gate holds whatever the row's
+    magnitude: fp32 rows of magnitude 1e4, 1e-3 and 1e-6 (unscaled, the remainders of the last
+    two would be fp16 subnormals or zero), a row with two entries beyond 65504 (which would be
+    infinities in fp16), and the same rows as bf16."""
+    N, K = 512, 1024
+    quants, meta_a, meta_b = engine.synth_q4_affine(91, 0.02, N, K, engine.META_BF16_PLANES)
+    base = make_x(engine, 92, 4, K, engine.F32)
+    x = np.stack([base[0] * np.float32(1e4), base[1] * np.float32(1e-3), base[2] * np.float32(1e-6), base[3]])
+    x[3, 5], x[3, 77] = np.float32(1e5), np.float32(-2.5e5)
+    x_bf = bf16_bits(x).reshape(4, K)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+    try:
+        print("activation range case", flush=True)
+        y = gpu.q4_linear(weight, x, engine.F32, engine.F32)
+        y_bf = gpu.q4_linear(weight, x_bf, engine.BF16, engine.F32)
+        y_one = gpu.q4_linear(weight, x[2:3], engine.F32, engine.F32)
+    finally:
+        weight.destroy()
+    assert np.all(np.isfinite(y)) and np.all(np.isfinite(y_bf))
+    ref = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x, engine.F32, 4)
+    assert q4_relative_error(y, ref) <= TOLERANCE
+    assert q4_relative_error(y_one, ref[2:3]) <= TOLERANCE
+    ref_bf = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x_bf, engine.BF16, 4)
+    assert q4_relative_error(y_bf, ref_bf) <= TOLERANCE
+
+
+SLICED_CASES = [
+    # name, [N per target], K, M, x dtype, fused gate-up-silu
+    ("small", [320], 8704, 8, "F16", False),
+    ("down_m1", [5120], 17408, 1, "F16", False),
+    ("down_m2", [5120], 17408, 2, "F16", False),
+    ("down_m4", [5120], 17408, 4, "F16", False),
+    ("down_m8", [5120], 17408, 8, "F16", False),
+    ("down_m4_f32", [5120], 17408, 4, "F32", False),
+    ("three_targets", [640, 320, 336], 8704, 8, "F16", False),
+    ("fused_silu", [640, 640], 8704, 8, "F16", True),
+]
+
+
+@pytest.mark.parametrize("name,rows,K,M,x_dtype,fused", SLICED_CASES, ids=[c[0] for c in SLICED_CASES])
+def test_slices_added_in_kernel_match_second_kernel(engine, oracle, gpu, name, rows, K, M, x_dtype, fused):
     """K slices are added by the last workgroup of a column to arrive, which needs the
     workgroups of a column on one XCD (probed when a context is created).  The probe must
-    say so on this GPU, and a context created with the in-kernel addition switched off (a
+    say so on this GPU, and the same context with the in-kernel addition switched off (a
     second kernel adds the slices) must give the same bits: both add in slice order.
-    Repeated calls (the arrival counters return to zero) stay bitwise equal too."""
+    Cases: the 27B down projection at every verify row count, fp32 activations (row pairs),
+    a sliced launch of three weights, and the fused gate-up-SiLU launch whose nonlinearity the
+    adding workgroup applies.  Repeated calls (the arrival counters return to zero) and a
+    recorded graph's replays stay bitwise equal too."""
     shared, xcds = gpu.probe_xcd_columns()
-    print(f"xcds={xcds} columns_share_xcd={shared}", flush=True)
+    print(f"sliced case {name}: xcds={xcds} columns_share_xcd={shared}", flush=True)
     assert shared and xcds >= 1
-    N, K, M = 320, 8704, 8
-    quants, meta_a, meta_b = engine.synth_q4_affine(41, 0.02, N, K, engine.META_BF16_PLANES)
-    x = make_x(engine, 42, M, K, engine.F16)
-    results = []
-    for off in (False, True):
-        if off:
-            monkeypatch.setenv("MI355Q_NO_ARRIVALS", "1")
-        ctx = engine.Context(0)
-        weight = ctx.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
-        try:
-            results.append([ctx.q4_linear(weight, x, engine.F16, engine.F32) for _ in range(3)])
-        finally:
-            weight.destroy()
-    ref = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x, engine.F16, M)
-    assert q4_relative_error(results[0][0], ref) <= TOLERANCE
-    for y in results[0] + results[1]:
-        assert np.array_equal(y.view(np.uint32), results[0][0].view(np.uint32))
+    x_dtype = getattr(engine, x_dtype)
+    kind = engine.META_BF16_PLANES
+    images = [engine.synth_q4_affine(41 + i, 0.02, N, K, kind) for i, N in enumerate(rows)]
+    x = make_x(engine, 42, M, K, x_dtype)
+    ctx = engine.Context(0)
+    weights = [ctx.q4_prepare(*image, N, K, kind) for image, N in zip(images, rows)]
+    pointers, graph = [], None
+    try:
+        x_ptr = ctx.to_device(x)
+        outputs = 1 if fused else len(rows)
+        y_ptr = [ctx.alloc(M * N * 4) for N in rows[:outputs]]
+        pointers = [x_ptr] + y_ptr
+        targets = [(w, y_ptr[i] if i < outputs else None) for i, w in enumerate(weights)]
+        calls = engine.make_calls([(targets, x_ptr, x_dtype, M, engine.F32, engine.F32,
+                                    engine.FUSE_GATE_UP_SILU if fused else 0)])
+
+        def run(launch):
+            for pointer, N in zip(y_ptr, rows):
+                ctx.upload(pointer, np.zeros((M, N), dtype=np.float32))
+            launch()
+            ctx.sync()
+            return [ctx.download(pointer, (M, N), np.float32) for pointer, N in zip(y_ptr, rows)]
+
+        ctx.set_option("trace", "1")
+        in_kernel = [run(lambda: ctx.q4_sequence(calls)) for _ in range(3)]
+        ctx.set_option("trace", None)
+        graph = ctx.q4_sequence_record(calls)
+        replays = [run(lambda: ctx.graph_launch(graph)) for _ in range(3)]
+        ctx.set_option("in_kernel_slices", "0")
+        second_kernel = [run(lambda: ctx.q4_sequence(calls)) for _ in range(2)]
+    finally:
+        if graph is not None:
+            ctx.graph_destroy(graph)
+        for pointer in pointers:
+            ctx.free(pointer)
+        for w in weights:
+            w.destroy()
+        ctx.close()
+    for label, runs in (("in-kernel", in_kernel), ("graph replay", replays), ("second kernel", second_kernel)):
+        for index, outputs_of_run in enumerate(runs):
+            for got, first in zip(outputs_of_run, in_kernel[0]):
+                assert np.array_equal(got.view(np.uint32), first.view(np.uint32)), f"{label} run {index}"
+    refs = [oracle.q4_linear(*image, kind, N, K, x, x_dtype, M) for image, N in zip(images, rows)]
+    if fused:
+        refs = [refs[0] / (1.0 + np.exp(-refs[0])) * refs[1]]
+    for got, ref in zip(in_kernel[0], refs):
+        assert q4_relative_error(got, ref) <= TOLERANCE
 
 
 def test_recorded_sequence_replays(engine, oracle, gpu):

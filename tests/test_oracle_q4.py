@@ -242,3 +242,25 @@ def test_q8_affine_matches_numpy_float64(oracle):
     seq = oracle.q8_affine_linear(quants, meta, None, oracle.META_F16_INTERLEAVED, N, K, x, oracle.X_F16, M,
                                   accumulate=oracle.ACC_F32_SEQUENTIAL)
     assert np.max(np.abs(seq - expect)) <= 1e-4 * np.max(np.abs(expect))
+
+
+def test_recipe_generators_agree(oracle):
+    """The C generator of the Qwen3.8 benchmark's xorshift32 matrices (used by the GPU tests at
+    full size) against the step-by-step numpy restatement of the same recipe on the first 700
+    groups of each seed, and the activation formula's first values against Python floats."""
+    import math
+
+    import recipes
+    for seed in recipes.QWEN38_SEEDS.values():
+        quants, meta = recipes.qwen38_weights(oracle, seed, 8, 5120)
+        slow_q, slow_m = recipes.qwen38_weights_numpy(seed, 640)
+        assert np.array_equal(quants, slow_q) and np.array_equal(meta, slow_m)
+    scales = meta[0::2].view(np.float16).astype(np.float32)
+    assert scales.min() >= 0.0035 - 1e-5 and scales.max() <= 0.0035 + 7 * 0.00025 + 1e-5
+    x = recipes.qwen38_activation(2, 5120)
+    for i in (0, 1, 77, 5119, 5120, 10239):
+        expect = 0.75 * math.sin(np.float32(0.013) * np.float32(i)) + 0.20 * math.cos(np.float32(0.031) * np.float32(i))
+        assert abs(float(x.reshape(-1)[i]) - expect) <= 1e-3
+    h3 = recipes.h3_input(2)
+    assert h3[0, 0] == np.float32(0.0625 * (17 % 17 - 8)) and h3[1, 0] == np.float32(0.0625 * ((13 * 5376 + 17) % 17 - 8))
+    assert set(np.unique(h3 * 16).astype(int)) <= set(range(-8, 9))

@@ -62,17 +62,47 @@ def test_live_reference_build(oracle):
     assert np.array_equal(out.view(np.uint32), expect.view(np.uint32))
 
 
-def test_weight_quantizer_properties(oracle):
-    """The reference's weight quantizer is Python (q8_payload) and is not executed: parity unpinned.
-    Checked here: the record layout, scale = max|w|/127 as fp32, |q| <= 127, ties to even, zero row."""
-    w = np.array([[0.0] * 8, [1.27, -1.27, 0.005, 0.015, 0.025, -0.005, 0.635, 0.0]], dtype=np.float32)
-    rows = oracle.q8_weight_quantize(w).reshape(2, 12)
-    assert rows[0, :4].view(np.float32)[0] == 1.0 and not rows[0, 4:].any()
-    scale = rows[1, :4].view(np.float32)[0]
-    assert scale == np.float32(np.float64(np.float32(1.27)) / 127.0)
-    q = rows[1, 4:].view(np.int8)
-    assert q[0] == 127 and q[1] == -127 and np.all(np.abs(q.astype(int)) <= 127)
-    assert np.array_equal(q, np.clip(np.rint(w[1] / scale), -127, 127).astype(np.int8))
+Q8_PAYLOAD_CASES = ("normal", "ties", "halves", "wide")
+
+
+@pytest.mark.parametrize("case", Q8_PAYLOAD_CASES)
+def test_weight_quantizer_matches_reference_payload_bytes(oracle, engine, case):
+    """orc_q8_weight_quantize and the library's host quantizer mi355q_quantize_w8_rows against the
+    record bytes the reference's own q8_payload produced (compile_minimindo_sensevoice_image.py:
+    38-46; tests/golden/q8_payload.npz, written by make_q8_payload_fixture.py): N(0,0.02) rows with
+    an all-zero and a constant row, quotients on and one float32 step beside every .5, exact
+    halves at scale 1, and row maxima from 1e-30 to 1e30 with subnormal entries.  Byte for byte."""
+    golden = np.load(GOLDEN.with_name("q8_payload.npz"), allow_pickle=False)
+    w, records = golden[f"{case}_w"], golden[f"{case}_records"]
+    N, K = w.shape
+    assert np.array_equal(oracle.q8_weight_quantize(w).reshape(-1), records)
+    mine = np.empty(N * (4 + K), dtype=np.uint8)
+    status = engine.library().mi355q_quantize_w8_rows(w.ctypes.data, N, K, mine.ctypes.data)
+    assert status == 0 and np.array_equal(mine, records)
+
+
+def test_reference_payload_fixture_tells_plausible_mistakes_apart():
+    """The fixture is only a pin if the likely wrong restatements disagree with it somewhere:
+    multiplying by 1/scale instead of dividing, rounding halves away from zero and dividing in
+    double each differ from the recorded bytes.  (max/127 computed in float32 or in double and
+    then rounded cannot differ: 1/127 has a binary period of seven bits, so no quotient of a
+    24-bit maximum sits close enough to a float32 midpoint for the second rounding to matter.)"""
+    golden = np.load(GOLDEN.with_name("q8_payload.npz"), allow_pickle=False)
+    wrong = {"reciprocal": 0, "half_away": 0, "double_division": 0}
+    for case in Q8_PAYLOAD_CASES:
+        w = golden[f"{case}_w"]
+        N, K = w.shape
+        records = golden[f"{case}_records"].reshape(N, 4 + K)
+        scale = records[:, :4].copy().view(np.float32).reshape(N)
+        q = records[:, 4:].view(np.int8)
+        maximum = np.abs(w).max(axis=1)
+        with np.errstate(all="ignore"):
+            wrong["reciprocal"] += int((np.clip(np.rint(w * (np.float32(1) / scale)[:, None]), -127, 127) != q).sum())
+            away = np.sign(w) * np.floor(np.abs(w / scale[:, None]) + np.float32(0.5))
+            wrong["half_away"] += int((np.clip(away, -127, 127) != q).sum())
+            in_double = np.rint(w.astype(np.float64) / (maximum.astype(np.float64) / 127.0)[:, None])
+            wrong["double_division"] += int((np.clip(np.nan_to_num(in_double), -127, 127) != q).sum())
+    assert all(count > 0 for count in wrong.values()), wrong
 
 
 def test_q8rows_f32_matches_reference_golden_bitwise(oracle):
