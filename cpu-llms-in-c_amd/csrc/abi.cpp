@@ -129,6 +129,7 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipEventCreate(&ctx->timer_stop);
     if (status == hipSuccess) status = hipMalloc((void **)&ctx->arrivals, kArrivalCounters * sizeof(uint32_t));
     if (status == hipSuccess) status = hipMemset(ctx->arrivals, 0, kArrivalCounters * sizeof(uint32_t));
+    if (status == hipSuccess) status = q4_stream_scratch_init(ctx);  // this device is current
     uint32_t xcds = 0;
     if (status == hipSuccess) status = probe_columns_share_xcd(ctx, &ctx->columns_share_xcd, &xcds);
     ctx->columns_probed = ctx->columns_share_xcd;
@@ -773,6 +774,54 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const 
     mi355q_q4_target target = {weight, y, residual};
     return mi355q_q4_linear_multi(ctx, &target, 1, x, x_dtype, M, y_dtype, residual_dtype, flags, error,
                                   error_capacity);
+}
+
+int mi355q_q4_linear_noalloc(mi355q_context *ctx, const mi355q_q4_weight *weight, const void *x,
+                             int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,
+                             int residual_dtype, uint32_t flags, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || weight == nullptr || x == nullptr || y == nullptr || M == 0 ||
+        !dtype_valid(x_dtype) || !dtype_valid(y_dtype) || (residual != nullptr && !dtype_valid(residual_dtype))) {
+        set_error(error, error_capacity, "q4_linear_noalloc: invalid argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (weight->ctx != ctx) {
+        set_error(error, error_capacity, "q4_linear_noalloc: weight belongs to another context");
+        return MI355Q_ERROR_INVALID;
+    }
+    if ((flags & ~(uint32_t)(MI355Q_ASYNC | MI355Q_RESIDUAL_IS_BIAS | MI355Q_X_DEVICE | MI355Q_Y_DEVICE |
+                             MI355Q_RESIDUAL_DEVICE)) != 0) {
+        set_error(error, error_capacity, "q4_linear_noalloc: flags 0x%x not supported here", flags);
+        return MI355Q_ERROR_INVALID;
+    }
+    const uint32_t rows = x_dtype == MI355Q_F32 ? 2u * M : M;
+    if (rows > 16u) {
+        set_error(error, error_capacity,
+                  "q4_linear_noalloc: at most 16 activation rows (8 of fp32), got %u", M);
+        return MI355Q_ERROR_INVALID;
+    }
+    if (((uintptr_t)x & 15u) != 0) {
+        set_error(error, error_capacity, "q4_linear_noalloc: x must be 16-byte aligned");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    Q4LinearArgs args;
+    memset(&args, 0, sizeof args);
+    args.x = x;
+    args.x_dtype = x_dtype;
+    args.M = M;
+    args.y_dtype = y_dtype;
+    args.residual_dtype = residual_dtype;
+    args.residual_is_bias = (flags & MI355Q_RESIDUAL_IS_BIAS) != 0;
+    args.count = 1;
+    args.targets[0].w = &weight->dev;
+    args.targets[0].y = y;
+    args.targets[0].residual = residual;
+    args.no_alloc = true;
+    const int status = q4_stream_linear(ctx, args, error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    if (!(flags & MI355Q_ASYNC)) MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear_noalloc sync");
+    return MI355Q_OK;
 }
 
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,

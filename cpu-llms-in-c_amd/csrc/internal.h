@@ -77,6 +77,9 @@ struct mi355q_context {
     int force_gemm[2];    // kernel variant, K splits; [1] == 0: no forcing
     bool trace;           // print the chosen decomposition of every launch to stderr
     bool lds_raised[16];  // q4_gemm_pipe_kernel instantiations whose dynamic LDS limit has been raised
+    // device address of the library's fixed scratch array on this context's device (for the
+    // entry point that allocates nothing); every context on the device sees the same array
+    unsigned char *fixed_scratch;
 };
 namespace mi355q {
 constexpr uint32_t kArrivalCounters = 65536;
@@ -168,7 +171,14 @@ struct Q4LinearArgs {
     uint32_t row_count;
     uint32_t count;
     Q4Target targets[kMaxTargets];
+    // The call may not allocate: converted activations, slice partial sums and arrival counters
+    // live in the library's fixed device array (q4_stream_scratch_init), sizes beyond it are
+    // refused, and so is per-kernel profiling (which creates events).
+    bool no_alloc;
 };
+// Looks up the device address of the fixed scratch array on the context's device (once per
+// device) and keeps it in the context; called by mi355q_context_create with that device current.
+hipError_t q4_stream_scratch_init(mi355q_context *ctx);
 int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity);
 // q4_gemm.hip (one target at a time: `target` selects it)
 int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,

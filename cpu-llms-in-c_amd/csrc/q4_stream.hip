@@ -30,12 +30,49 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
 namespace mi355q {
 
-constexpr size_t kRowScaleBytes = 256;  // one float per activation row in front of converted rows
+// ---- fixed scratch for the entry point that allocates nothing -----------------------------
+// One array per GPU, held from the moment the library's code object is loaded on it until the
+// process ends: [ converted activations | slice partial sums | arrival counters ].  In host
+// code the array's name is only a handle for hipGetSymbolAddress; kernels and fills get the
+// device address that call returns (kept per device below and in every context).
+constexpr size_t kRowScaleBytes = 256;              // one float per activation row in front of converted rows
+constexpr size_t kScratchXBytes = 1u << 20;         // converted activations: 256 + rows * K * 2 bytes
+constexpr size_t kScratchPartialBytes = 2u << 20;   // fp32 partial sums: slices * M * N_total * 4 bytes
+constexpr uint32_t kScratchCounters = 4096;         // arrival counters (workgroup columns + 8)
+constexpr size_t kScratchBytes = kScratchXBytes + kScratchPartialBytes + kScratchCounters * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static unsigned char *scratch_on_device[kMaxDevices];  // written once per device, under the lock
+static std::mutex scratch_lock;
+
+hipError_t q4_stream_scratch_init(mi355q_context *ctx)
+{
+    if (ctx->device < 0 || ctx->device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (scratch_on_device[ctx->device] == nullptr) {
+        void *address = nullptr;
+        const hipError_t status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (status != hipSuccess) return status;
+        if (address == nullptr) return hipErrorInvalidSymbol;
+        scratch_on_device[ctx->device] = (unsigned char *)address;
+    }
+    ctx->fixed_scratch = scratch_on_device[ctx->device];
+    return hipSuccess;
+}
+
+// sets `count` 32-bit words to zero (a kernel, not a memset node: callers may be recording a graph)
+__global__ void __launch_bounds__(256) zero_words_kernel(uint32_t *words, uint32_t count)
+{
+    const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
+    if (index < count) words[index] = 0u;
+}
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
 // compile-time constant in the body
@@ -733,12 +770,27 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     StreamParams p;
     memset(&p, 0, sizeof p);
     p.x = (const _Float16 *)a.x;
+    if (a.no_alloc && (ctx->fixed_scratch == nullptr || ctx->profiling)) {
+        set_error(error, error_capacity, "q4 stream kernel: the non-allocating call needs the fixed scratch "
+                                         "array and cannot run under per-kernel profiling");
+        return MI355Q_ERROR_INVALID;
+    }
     if (a.x_dtype != MI355Q_F16) {
         // [ the rows' inverse scales (16 floats, 256 bytes) | rows * K fp16 ]
         const size_t bytes = kRowScaleBytes + (size_t)rows * first.K * sizeof(_Float16);
-        int status = ensure_stage(ctx, 3, bytes, error, error_capacity);
-        if (status != MI355Q_OK) return status;
-        unsigned char *const area = (unsigned char *)ctx->stage[3];
+        unsigned char *area;
+        if (a.no_alloc) {
+            if (bytes > kScratchXBytes) {
+                set_error(error, error_capacity, "non-allocating call: %zu bytes of converted activations "
+                                                 "(256 + rows * K * 2) exceed the fixed %zu", bytes, kScratchXBytes);
+                return MI355Q_ERROR_INVALID;
+            }
+            area = ctx->fixed_scratch;
+        } else {
+            int status = ensure_stage(ctx, 3, bytes, error, error_capacity);
+            if (status != MI355Q_OK) return status;
+            area = (unsigned char *)ctx->stage[3];
+        }
         float *const row_scale = (float *)area;
         _Float16 *const converted_x = (_Float16 *)(area + kRowScaleBytes);
         hipError_t converted = launch(ctx, q4_convert_x_kernel, dim3(a.M), dim3(kConvertThreads), 0, a.x,
@@ -795,10 +847,30 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         const size_t partial_bytes = (size_t)p.slices * a.M * p.n_total * sizeof(float);
         // grid.x of the launch: the workgroup columns that count arrivals
         const uint32_t columns = a.fuse_silu ? (p.NT[0] + shape.tb / 2 - 1) / (shape.tb / 2) : block;
-        int status = ensure_stage(ctx, 4, partial_bytes, error, error_capacity);
-        if (status != MI355Q_OK) return status;
-        p.partials = (float *)ctx->stage[4];
-        p.arrivals = ctx->columns_share_xcd && columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
+        if (a.no_alloc) {
+            if (partial_bytes > kScratchPartialBytes) {
+                set_error(error, error_capacity, "non-allocating call: %zu bytes of slice partial sums "
+                                                 "(slices * M * N * 4) exceed the fixed %zu", partial_bytes,
+                          kScratchPartialBytes);
+                return MI355Q_ERROR_INVALID;
+            }
+            p.partials = (float *)(ctx->fixed_scratch + kScratchXBytes);
+            uint32_t *const counters = (uint32_t *)(ctx->fixed_scratch + kScratchXBytes + kScratchPartialBytes);
+            p.arrivals = ctx->columns_share_xcd && columns + 8u <= kScratchCounters ? counters : nullptr;
+            if (p.arrivals) {
+                // the array is shared by every call on this GPU and keeps what the last one left:
+                // the counters this launch uses start from zero whatever happened before
+                const uint32_t used = (columns + 7u) / 8u * 8u;
+                hipError_t zeroed = launch(ctx, zero_words_kernel, dim3((used + 255u) / 256u), dim3(256), 0,
+                                           counters, used);
+                if (zeroed != hipSuccess) return fail_hip(zeroed, "arrival counter reset", error, error_capacity);
+            }
+        } else {
+            int status = ensure_stage(ctx, 4, partial_bytes, error, error_capacity);
+            if (status != MI355Q_OK) return status;
+            p.partials = (float *)ctx->stage[4];
+            p.arrivals = ctx->columns_share_xcd && columns + 8u <= kArrivalCounters ? ctx->arrivals : nullptr;
+        }
     }
     p.pair = pair;
     p.y_dtype = a.y_dtype;

@@ -103,6 +103,7 @@ SIGNATURES = {
     "mi355q_q4_dequant_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_rows": (_int, [_vp, _vp, _vp, _u32, _vp, _int, _u32, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
+    "mi355q_q4_linear_noalloc": (_int, [_vp, _vp, _vp, _int, _u32, _vp, _int, _vp, _int, _u32, *_err]),
     "mi355q_q4_linear_multi": (_int, [_vp, _c.POINTER(Q4Target), _u32, _vp, _int, _u32, _int, _int,
                                       _u32, *_err]),
     "mi355q_q4_linear_sequence": (_int, [_vp, _c.POINTER(Q4Call), _sz, *_err]),
@@ -435,6 +436,14 @@ class Context:
                          residual_dtype: int = F32, asynchronous: bool = True):
         flags = X_DEVICE | Y_DEVICE | RESIDUAL_DEVICE | (ASYNC if asynchronous else 0)
         _call(self.lib.mi355q_q4_linear, self.handle, weight.handle, x_ptr, x_dtype, M, y_ptr,
+              y_dtype, residual_ptr, residual_dtype, flags)
+
+    def q4_linear_noalloc(self, weight: Q4Weight, x_ptr: int, x_dtype: int, M: int, y_ptr: int,
+                          y_dtype: int, residual_ptr: int | None = None, residual_dtype: int = F32,
+                          asynchronous: bool = False, residual_is_bias: bool = False):
+        """The entry point that allocates nothing; device pointers only."""
+        flags = (ASYNC if asynchronous else 0) | (RESIDUAL_IS_BIAS if residual_is_bias else 0)
+        _call(self.lib.mi355q_q4_linear_noalloc, self.handle, weight.handle, x_ptr, x_dtype, M, y_ptr,
               y_dtype, residual_ptr, residual_dtype, flags)
 
     # ---- W8A8 ----

@@ -333,6 +333,28 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight,
                      const void *residual, int residual_dtype,
                      uint32_t flags, char *error, size_t error_capacity);
 
+/* mi355q_q4_linear for callers that cannot allocate device memory while they run: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid it.  No counterpart in
+ * the reference.  Same result as mi355q_q4_linear, bit for bit (same kernels, same launch
+ * shapes), for 1..16 activation rows (8 of fp32); x, y and residual are DEVICE pointers
+ * (the *_DEVICE flags are implied), x 16-byte aligned.  It calls no hipMalloc / hipFree
+ * and no other allocating routine: what the ordinary call keeps in growable staging
+ * buffers — activations converted to fp16 (bf16 / fp32 x), the fp32 partial sums of K
+ * slices, their arrival counters — lives in one fixed array of 3 MiB + 16 KiB that the library
+ * holds on every GPU it is loaded on until the process ends.  Limits (status 2 beyond
+ * them): 256 + rows * K * 2 <= 1 MiB for x that is not fp16 (rows = 2 M for fp32), and
+ * slices * M * N * 4 <= 2 MiB when the launch is cut in K slices (the 27B down projection
+ * at M = 16: 0.94 MiB).  Refused (status 2) while mi355q_profile_begin is active.
+ * Flags: MI355Q_ASYNC, MI355Q_RESIDUAL_IS_BIAS.  All calls on one GPU share the array,
+ * which keeps what the last call left (the counters a launch uses are cleared by a small
+ * kernel in front of it): two such calls in flight at once on one GPU — two contexts, two
+ * threads — race on it; serialise them. */
+int mi355q_q4_linear_noalloc(mi355q_context *ctx, const mi355q_q4_weight *weight,
+                             const void *x, int x_dtype, uint32_t M,
+                             void *y, int y_dtype,
+                             const void *residual, int residual_dtype,
+                             uint32_t flags, char *error, size_t error_capacity);
+
 /* One activation matrix against up to four weights that share K and the
  * metadata kind, in ONE kernel launch for M <= 16: y_t = x * w_t^T (+ residual_t).
  * This is how a decoder layer uses the path — q, k and v read the same x, and
