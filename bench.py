@@ -7,27 +7,33 @@ up 5120->17408, down 17408->5120 — in affine-Q4 group-64 with bf16 scale/bias,
 fp16 activations and fp16 outputs, on seeded synthetic weights (N(0,0.02)
 before quantization) and activations (N(0,1)).  One step is one pass over the
 seven linears of one weight copy (four launches: q|k|v and gate|up share their
-activations and go out as one launch each, then o and down); successive steps rotate over `--copies`
-distinct prepared copies (>= 1.5 GB in total) so that the 256 MB memory-side
-cache cannot serve the weights and the figure is an HBM figure.
+activations and go out as one launch each, then o and down); successive steps
+rotate over `--copies` distinct prepared copies (>= 1.5 GB in total) so that the
+256 MB memory-side cache cannot serve the weights and the figure is an HBM figure.
 
 Prints ONE JSON line.  `value` is algorithmic bytes (N*K/2 + N*(K/64)*4 +
 M*K*2 + M*N*2 per linear) per second of wall time over the timed steps, with
 all inputs resident in HBM before the clock starts.  `roofline` prices the
 dominant kernel (the weight-streaming Q4 kernel) against HBM: algorithmic bytes
 per launch over the kernel's own average duration (HIP events bound to each
-dispatch, measured in a second pass of the same steps).  `cpu_baseline` is the
+dispatch, measured in a second pass of the same steps).  Before anything is
+timed the GPU runs the same steps untimed until at least `--preheat-ms` of GPU
+time have passed (clocks and power state settle; `config.preheat_ms` says how
+long it ran): a 20-step run then reads like a 400-step run.  `cpu_baseline` is the
 CPU oracle (a C restatement of the reference's scalar loop, row-parallel with
 OpenMP as the reference parallelises its GEMV) timed on this host on the same
-layer.
+layer, with the CPU model, the threads used and the host's read bandwidth.
+
+The default line also carries `secondary`: the other configurations of the
+headline metric, each measured briefly in the same process on the same weights —
+the speculative-verify batches (M = 2, 4, 8: HBM roofline), the prefill GEMMs of
+the MLP at M = 512 (gate, up, down: fp16 matrix-instruction roofline) and the
+W8A8 encoder projections (M=64, K=1024, N=4096: int8 roofline, accumulators
+compared bit for bit with the CPU oracle).  `--no-secondary` leaves them out.
 
 Other workloads (never the default; each prints its own JSON line of the same
-shape): `--workload prefill --rows 512` times the gate, up and down GEMMs of the
-same layer at M rows against the fp16 matrix-instruction peak (2*M*K*N flops per
-linear); `--workload w8a8` times one activation quantization and the three
-projections that share it (M=64, K=1024, N=4096) in int8 with int32
-accumulators, and checks the accumulators bit for bit against the CPU oracle in
-the cpu_baseline leg; `--rows 2..8` turns the default workload into the
+shape): `--workload prefill --rows 512`, `--workload w8a8`, `--workload lm_head`,
+`--workload config1`; `--rows 2..8` turns the default workload into the
 small-M verify case.
 """
 from __future__ import annotations
@@ -72,91 +78,62 @@ def q4_bytes(N, K, M, y_bytes=2):
     return N * K // 2 + N * (K // 64) * 4 + M * K * 2 + M * N * y_bytes
 
 
-def build_workload(engine, ctx, shapes, M, copies, meta_kind, verbose, fuse=True, silu=False):
-    """Prepares `copies` device copies of every matrix plus activations/outputs."""
-    x_ptr, y_ptr, weights, host = {}, {}, [[] for _ in range(copies)], {}
-    for index, (name, N, K) in enumerate(shapes):
-        t0 = time.perf_counter()
-        quants, meta_a, meta_b = engine.synth_q4_affine(1000 + index, 0.02, N, K, meta_kind)
-        host[name] = (quants, meta_a, meta_b)
-        for copy in range(copies):
-            weights[copy].append(ctx.q4_prepare(quants, meta_a, meta_b, N, K, meta_kind))
-        if K not in x_ptr:
-            rows = [engine.synth_normal_f16(77 + 1000 * m + K, 1.0, K) for m in range(M)]
-            host[("x", K)] = np.stack(rows)
-            x_ptr[K] = ctx.to_device(host[("x", K)])
-        y_ptr[name] = ctx.alloc(max(M * N * 2, 16))
-        if verbose:
-            print(f"# prepared {name} {N}x{K} x{copies} in {time.perf_counter() - t0:.2f}s",
-                  file=sys.stderr, flush=True)
-    calls = []
-    for copy in range(copies):
-        # linears that read the same activations go out as one launch (q|k|v, gate|up)
-        groups = []
-        for i, (name, N, K) in enumerate(shapes):
-            target = (weights[copy][i], y_ptr[name])
-            share = fuse and groups and groups[-1][1] == K and name.split("_")[0] in ("k", "v", "up")
-            if share:
-                groups[-1][0].append(target)
-            else:
-                groups.append(([target], K))
-        # --fused-mlp: the gate|up launch writes silu(gate . x) * (up . x) into gate's output
-        calls.append(engine.make_calls([
-            (targets, x_ptr[K], engine.F16, M, engine.F16, engine.F32,
-             engine.FUSE_GATE_UP_SILU if silu and len(targets) == 2 else 0)
-            for targets, K in groups]))
-    return calls, weights, host, x_ptr, y_ptr
+# ---- host context ------------------------------------------------------------------------------
+
+def host_threads():
+    """Threads for the CPU baseline: every CPU this process may run on, but no more than the job's
+    share when the launcher has set one (OMP_NUM_THREADS)."""
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    threads = min(allowed, int(cap)) if cap.isdigit() and int(cap) > 0 else allowed
+    return max(threads, 1), allowed
 
 
-def weights_digest(host, shapes):
-    """SHA-256 over the packed synthetic weights (codes, then metadata planes, matrix by matrix)."""
-    import hashlib
-    digest = hashlib.sha256()
-    for name, _, _ in shapes:
-        for plane in host[name]:
-            if plane is not None:
-                digest.update(np.ascontiguousarray(plane).view(np.uint8))
-    return digest.hexdigest()
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as stream:
+            for line in stream:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
-def cpu_baseline(oracle, shapes, host, M, meta_kind, budget_s=10.0):
-    """The oracle's reference-faithful flavour (fp32, k order) on all host threads: passes over
-    the layer for about `budget_s` seconds (at least 5, at most 200), the median taken."""
-    threads = min(os.cpu_count() or 1, 16)
-    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
-    total_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
-    times, repeats, rep = [], 5, 0
-    while rep < repeats + 1:
-        t0 = time.perf_counter()
-        for name, N, K in shapes:
-            quants, meta_a, meta_b = host[name]
-            oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, host[("x", K)], oracle.X_F16,
-                             M, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=threads)
-        if rep:
-            times.append(time.perf_counter() - t0)
-        if rep == 1:  # the first pass warms up; the second sizes the sample
-            repeats = max(5, min(200, int(budget_s / max(times[0], 1e-4))))
-        rep += 1
-    median = sorted(times)[len(times) // 2]
-    t0 = time.perf_counter()  # the reference's deployment width: four threads (one pass)
-    for name, N, K in shapes:
-        quants, meta_a, meta_b = host[name]
-        oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, host[("x", K)], oracle.X_F16,
-                         M, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=4)
-    four = time.perf_counter() - t0
+def host_fields(oracle, threads, allowed):
+    """CPU model, thread counts and the host's read bandwidth at 1 and `threads` threads (the
+    reference's target-probe measurement, tools/target_probe.c)."""
     return {
-        "value": round(total_bytes / median / 1e9, 3),
-        "value_at_4_threads": round(total_bytes / four / 1e9, 3),
-        "unit": "GB/s",
+        "cpu_model": cpu_model(),
         "cores": threads,
-        "kind": "port",
-        "sample": f"{repeats} passes over the same layer (median), oracle restatement of "
-                  f"cpu_row_dot, OpenMP static over rows, {median * 1e3:.1f} ms per pass",
+        "host_cpus_online": os.cpu_count(),
+        "host_cpus_allowed": allowed,
+        "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
+        "host_read_gib_per_s": {"threads_1": round(oracle.probe_read_gib_per_s(threads=1, seconds=0.4), 2),
+                                "threads_%d" % threads: round(oracle.probe_read_gib_per_s(threads=threads,
+                                                                                         seconds=0.4), 2)},
     }
 
-def time_steps(ctx, run_steps, steps, warmup):
+
+# ---- timing helpers ----------------------------------------------------------------------------
+
+def preheat(ctx, run_steps, minimum_ms, batch):
+    """Runs steps untimed until `minimum_ms` of GPU time have passed; returns the GPU ms it took."""
+    total = 0.0
+    while total < minimum_ms:
+        ctx.timer_begin()
+        run_steps(batch)
+        total += ctx.timer_end()
+    return total
+
+
+def time_steps(ctx, run_steps, steps, warmup, preheat_ms=0.0, preheat_batch=50):
     """Wall and event time of `steps` steps after `warmup`, then the same steps again with an
-    event pair around every dispatch: (wall s, gpu ms, sum of kernel ms, kernel launches)."""
+    event pair around every dispatch: dict(wall s, gpu ms, kernel ms, launches, per-launch us)."""
+    heated = preheat(ctx, run_steps, preheat_ms, preheat_batch) if preheat_ms > 0 else 0.0
     run_steps(warmup)
     ctx.sync()
     t0 = time.perf_counter()
@@ -165,10 +142,16 @@ def time_steps(ctx, run_steps, steps, warmup):
     gpu_ms = ctx.timer_end()  # waits for the stream
     ctx.sync()
     wall = time.perf_counter() - t0
+    # per-dispatch pass: the warm-up steps run in the same mode first (it launches through another
+    # runtime call and creates its events on first use), then the counted steps follow at once
+    ctx.profile_begin()
+    run_steps(max(warmup, 2))
+    ctx.profile_end()
     ctx.profile_begin()
     run_steps(steps)
     kernel_ms, launches = ctx.profile_end()
-    return wall, gpu_ms, kernel_ms, launches
+    return {"wall": wall, "gpu_ms": gpu_ms, "kernel_ms": kernel_ms, "launches": int(launches),
+            "per_launch_us": ctx.profile_durations(), "preheat_ms": heated}
 
 
 def common_fields(args, wall):
@@ -184,25 +167,183 @@ def common_fields(args, wall):
 
 
 def device_fields(info):
-    return {"device": info.name.decode(errors="replace").strip(),
-            "arch": info.arch.decode(errors="replace"),
+    name = info.name.decode(errors="replace").strip()
+    arch = info.arch.decode(errors="replace")
+    return {"device": name or "(the runtime reports no product name; arch %s)" % arch,
+            "arch": arch,
             "max_clock_mhz": info.clock_mhz, "memory_clock_mhz": info.memory_clock_mhz,
             "memory_bus_bits": info.memory_bus_bits, "compute_units": info.compute_units}
 
 
-def bench_prefill(engine, ctx, args):
-    """gate, up (one call, shared activations) and down at M rows: fp16 matrix-instruction GEMMs."""
-    M = args.rows
-    copies = 2
+# ---- Q4 layer workloads ------------------------------------------------------------------------
+
+class LayerWorkload:
+    """`copies` prepared device copies of every matrix of `shapes` plus activations/outputs."""
+
+    def __init__(self, engine, ctx, shapes, copies, meta_kind, max_rows, verbose=False):
+        self.engine, self.ctx, self.shapes, self.copies, self.meta_kind = engine, ctx, shapes, copies, meta_kind
+        self.host, self.weights, self.x_ptr, self.y_ptr = {}, [[] for _ in range(copies)], {}, {}
+        for index, (name, N, K) in enumerate(shapes):
+            t0 = time.perf_counter()
+            self.host[name] = engine.synth_q4_affine(1000 + index, 0.02, N, K, meta_kind)
+            for copy in range(copies):
+                self.weights[copy].append(ctx.q4_prepare(*self.host[name], N, K, meta_kind))
+            if K not in self.x_ptr:
+                rows = [engine.synth_normal_f16(77 + 1000 * m + K, 1.0, K) for m in range(max_rows)]
+                self.host[("x", K)] = np.stack(rows)
+                self.x_ptr[K] = ctx.to_device(self.host[("x", K)])
+            self.y_ptr[name] = ctx.alloc(max(max_rows * N * 2, 16))
+            if verbose:
+                print(f"# prepared {name} {N}x{K} x{copies} in {time.perf_counter() - t0:.2f}s",
+                      file=sys.stderr, flush=True)
+
+    def calls(self, M, fuse=True, silu=False):
+        """One call array per copy: linears that read the same activations go out as one launch
+        (q|k|v, gate|up); rows 0..M-1 of the activations."""
+        engine, out = self.engine, []
+        for copy in range(self.copies):
+            groups = []
+            for i, (name, N, K) in enumerate(self.shapes):
+                target = (self.weights[copy][i], self.y_ptr[name])
+                share = fuse and groups and groups[-1][1] == K and name.split("_")[0] in ("k", "v", "up")
+                if share:
+                    groups[-1][0].append(target)
+                else:
+                    groups.append(([target], K))
+            out.append(engine.make_calls([
+                (targets, self.x_ptr[K], engine.F16, M, engine.F16, engine.F32,
+                 engine.FUSE_GATE_UP_SILU if silu and len(targets) == 2 else 0)
+                for targets, K in groups]))
+        return out
+
+    def digest(self):
+        """SHA-256 over the packed synthetic weights (codes, then metadata planes, matrix by matrix)."""
+        import hashlib
+        digest = hashlib.sha256()
+        for name, _, _ in self.shapes:
+            for plane in self.host[name]:
+                if plane is not None:
+                    digest.update(np.ascontiguousarray(plane).view(np.uint8))
+        return digest.hexdigest()
+
+    def destroy(self):
+        for copy in self.weights:
+            for weight in copy:
+                weight.destroy()
+
+
+def measure_layer(ctx, work, M, steps, warmup, preheat_ms, fuse=True, silu=False, graph=False):
+    """Times `steps` layer steps at M rows; returns the figures of one layer line."""
+    calls = work.calls(M, fuse=fuse, silu=silu)
+    copies = work.copies
+    launches_per_step = len(calls[0])
+    step_bytes = sum(q4_bytes(N, K, M) for _, N, K in work.shapes)
+
+    def run_steps(count):
+        for step in range(count):
+            ctx.q4_sequence(calls[step % copies])
+
+    graphs = [ctx.q4_sequence_record(c) for c in calls] if graph else None
+
+    def run_timed(count):
+        if graphs is None:
+            return run_steps(count)
+        for step in range(count):
+            ctx.graph_launch(graphs[step % copies])
+
+    heated = preheat(ctx, run_timed, preheat_ms, 100) if preheat_ms > 0 else 0.0
+    run_timed(warmup)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_begin()
+    run_timed(steps)
+    gpu_ms = ctx.timer_end()  # waits for the stream
+    ctx.sync()
+    wall = time.perf_counter() - t0
+
+    # second pass of the same steps with an event pair bound to every dispatch (after the
+    # warm-up steps in the same mode, see time_steps)
+    ctx.profile_begin()
+    run_steps(max(warmup, 2))
+    ctx.profile_end()
+    ctx.profile_begin()
+    run_steps(steps)
+    kernel_ms, launches = ctx.profile_end()
+    per_launch = ctx.profile_durations()
+    for g in graphs or []:
+        ctx.graph_destroy(g)
+    # kernel time of each step (its launches, and the slice reductions some of them carry)
+    per_step = per_launch[:len(per_launch) // steps * steps].reshape(steps, -1).sum(axis=1)
+    p10, p50, p90 = (float(np.percentile(per_step, q)) for q in (10, 50, 90))
+    launch_p50 = None  # median duration of each launch of a step, in launch order
+    if len(per_launch) == steps * launches_per_step:
+        launch_p50 = [round(float(v), 2) for v in np.median(per_launch.reshape(steps, launches_per_step), axis=0)]
+    bytes_per_launch = step_bytes / launches_per_step
+    avg_kernel_us = kernel_ms * 1e3 / max(launches, 1)
+    return {
+        "calls": calls, "run_steps": run_steps, "wall": wall, "gpu_ms": gpu_ms, "preheat_ms": heated,
+        "step_bytes": step_bytes, "launches_per_step": launches_per_step, "launches": int(launches),
+        "value": step_bytes * steps / wall / 1e9,
+        "kernel_us_per_step": (p10, p50, p90), "launch_p50": launch_p50,
+        "bytes_per_launch": bytes_per_launch, "avg_kernel_us": avg_kernel_us,
+        "achieved": bytes_per_launch / (avg_kernel_us * 1e-6) / 1e9,
+    }
+
+
+def cpu_baseline_layer(oracle, shapes, host, M, meta_kind, budget_s=10.0):
+    """The oracle's reference-faithful flavour (fp32, k order) on the host's threads: passes over
+    the layer for about `budget_s` seconds (at least 5, at most 200), the median taken."""
+    threads, allowed = host_threads()
+    total_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
+
+    def one_pass(count):
+        t0 = time.perf_counter()
+        for name, N, K in shapes:
+            quants, meta_a, meta_b = host[name]
+            oracle.q4_linear(quants, meta_a, meta_b, meta_kind, N, K, host[("x", K)][:M], oracle.X_F16,
+                             M, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=count)
+        return time.perf_counter() - t0
+
+    times, repeats, rep = [], 5, 0
+    while rep < repeats + 1:
+        seconds = one_pass(threads)
+        if rep:
+            times.append(seconds)
+        if rep == 1:  # the first pass warms up; the second sizes the sample
+            repeats = max(5, min(200, int(budget_s / max(times[0], 1e-4))))
+        rep += 1
+    median = sorted(times)[len(times) // 2]
+    four = one_pass(4)  # the reference's deployment width: four threads (one pass)
+    return {
+        "value": round(total_bytes / median / 1e9, 3),
+        "value_at_4_threads": round(total_bytes / four / 1e9, 3),
+        "unit": "GB/s",
+        **host_fields(oracle, threads, allowed),
+        "kind": "port",
+        "sample": f"{repeats} passes over the same layer (median), oracle restatement of "
+                  f"cpu_row_dot, OpenMP static over rows, {median * 1e3:.1f} ms per pass",
+    }
+
+
+# ---- prefill -----------------------------------------------------------------------------------
+
+def measure_prefill(engine, ctx, M, steps, warmup, preheat_ms, weights=None, host=None, with_cpu=True):
+    """gate, up (one call, shared activations) and down at M rows: fp16 matrix-instruction GEMMs.
+    `weights`: per copy [gate, up, down] prepared weights to reuse (and `host` their images)."""
     meta_kind = engine.META_BF16_PLANES
-    weights, host, x_ptr, y_ptr = [[] for _ in range(copies)], {}, {}, {}
-    for index, (name, N, K) in enumerate(PREFILL):
-        host[name] = engine.synth_q4_affine(1004 + index, 0.02, N, K, meta_kind)
-        for copy in range(copies):
-            weights[copy].append(ctx.q4_prepare(*host[name], N, K, meta_kind))
+    own = weights is None
+    if own:
+        weights, host = [[] for _ in range(2)], {}
+        for index, (name, N, K) in enumerate(PREFILL):
+            host[name] = engine.synth_q4_affine(1004 + index, 0.02, N, K, meta_kind)
+            for copy in range(2):
+                weights[copy].append(ctx.q4_prepare(*host[name], N, K, meta_kind))
+    copies = len(weights)
+    x_host, x_ptr, y_ptr = {}, {}, {}
+    for name, N, K in PREFILL:
         if K not in x_ptr:
-            host[("x", K)] = engine.synth_normal_f16(77 + K, 1.0, M * K).reshape(M, K)
-            x_ptr[K] = ctx.to_device(host[("x", K)])
+            x_host[K] = engine.synth_normal_f16(77 + K, 1.0, M * K).reshape(M, K)
+            x_ptr[K] = ctx.to_device(x_host[K])
         y_ptr[name] = ctx.alloc(M * N * 2)
     calls = []
     for copy in range(copies):
@@ -215,32 +356,17 @@ def bench_prefill(engine, ctx, args):
         for step in range(count):
             ctx.q4_sequence(calls[step % copies])
 
-    wall, gpu_ms, kernel_ms, launches = time_steps(ctx, run_steps, args.steps, args.warmup)
+    timed = time_steps(ctx, run_steps, steps, warmup, preheat_ms, preheat_batch=10)
     step_flops = sum(2.0 * M * N * K for _, N, K in PREFILL)
-    value = step_flops * args.steps / wall / 1e12
-    achieved = step_flops * args.steps / (kernel_ms * 1e-3) / 1e12
+    value = step_flops * steps / timed["wall"] / 1e12
+    achieved = step_flops * steps / (timed["kernel_ms"] * 1e-3) / 1e12
+    # kernel time per linear: launches of a step in order are gate, up, down (+ a reduction kernel
+    # behind any of them that is cut in K splits)
     result = {
-        "metric": "q4_prefill_tflops_m%d_27b_mlp" % M,
-        "value": round(value, 2),
-        "unit": "TFLOP/s",
-        **common_fields(args, wall),
-        "dtype": "u4 codes dequantized to f16, f16 matrix instructions, f32 accumulate",
-        "data": "synthetic (seeded N(0,0.02) weights min/max-quantized to affine-Q4 g64, N(0,1) "
-                "fp16 activations)",
-        "config": {
-            "workload": "27B-shaped MLP linears gate/up (5120->17408) and down (17408->5120) at M=%d, "
-                        "affine-Q4 g64, bf16 scale+bias, fp16 x and y" % M,
-            "linears_per_step": 3,
-            "algorithmic_flops_per_step": step_flops,
-            "percent_of_f16_peak": round(100.0 * value / F16_MFMA_PEAK_TFLOPS, 2),
-            # what the matrix instruction sustains here from registers: alone, and with two or
-            # three packed-fp16 vector instructions per matrix instruction (in-register dequantization)
-            "measured_mfma_tflops": {"alone": round(ctx.probe_mfma_rate(0), 1),
-                                     "with_2_valu": round(ctx.probe_mfma_rate(2), 1),
-                                     "with_3_valu": round(ctx.probe_mfma_rate(3), 1)},
-            "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
-            **device_fields(ctx.info()),
-        },
+        "tflops": round(value, 2),
+        "percent_of_f16_peak": round(100.0 * value / F16_MFMA_PEAK_TFLOPS, 2),
+        "wall": timed["wall"], "gpu_ms": timed["gpu_ms"], "preheat_ms": round(timed["preheat_ms"], 1),
+        "step_flops": step_flops,
         "roofline": {
             "bound": "mfma",
             "achieved": round(achieved, 2),
@@ -248,19 +374,20 @@ def bench_prefill(engine, ctx, args):
             "unit": "TFLOP/s",
             "frac": round(achieved / F16_MFMA_PEAK_TFLOPS, 4),
             "traffic": None,
-            "kernel": "q4_gemm_kernel (with its split-K reduction where one runs)",
-            "launches": int(launches),
-            "kernel_us_per_linear": round(kernel_ms * 1e3 / (3 * args.steps), 3),
+            "kernel": "q4_gemm_pipe_kernel (with the K-split reduction where one runs)",
+            "launches": timed["launches"],
+            "kernel_us_per_linear": round(timed["kernel_ms"] * 1e3 / (3 * steps), 3),
+            "kernel_us_per_step": round(timed["kernel_ms"] * 1e3 / steps, 3),
             "algorithmic_flops_per_linear": step_flops / 3,
         },
     }
-    if not args.no_cpu:
+    if with_cpu:
         import oracle  # test infrastructure, used here only as the timed CPU baseline
-        threads = min(os.cpu_count() or 1, 16)
+        threads, allowed = host_threads()
         rows = min(M, 4)  # bounded sample: the first rows of the same activations
         t0 = time.perf_counter()
         for name, N, K in PREFILL:
-            oracle.q4_linear(*host[name], meta_kind, N, K, host[("x", K)][:rows], oracle.X_F16, rows,
+            oracle.q4_linear(*host[name], meta_kind, N, K, x_host[K][:rows], oracle.X_F16, rows,
                              oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=threads)
         seconds = time.perf_counter() - t0
         result["cpu_baseline"] = {
@@ -268,14 +395,52 @@ def bench_prefill(engine, ctx, args):
             "cores": threads, "kind": "port",
             "sample": "the first %d of the %d rows through the three linears, oracle restatement of "
                       "cpu_row_dot, OpenMP static over output rows, %.2f s" % (rows, M, seconds)}
+    for pointer in list(x_ptr.values()) + list(y_ptr.values()):
+        ctx.free(pointer)
+    if own:
+        for copy in weights:
+            for weight in copy:
+                weight.destroy()
+    return result
+
+
+def bench_prefill(engine, ctx, args):
+    M = args.rows
+    r = measure_prefill(engine, ctx, M, args.steps, args.warmup, args.preheat_ms, with_cpu=not args.no_cpu)
+    result = {
+        "metric": "q4_prefill_tflops_m%d_27b_mlp" % M,
+        "value": r["tflops"],
+        "unit": "TFLOP/s",
+        **common_fields(args, r["wall"]),
+        "dtype": "u4 codes dequantized to f16, f16 matrix instructions, f32 accumulate",
+        "data": "synthetic (seeded N(0,0.02) weights min/max-quantized to affine-Q4 g64, N(0,1) "
+                "fp16 activations)",
+        "config": {
+            "workload": "27B-shaped MLP linears gate/up (5120->17408) and down (17408->5120) at M=%d, "
+                        "affine-Q4 g64, bf16 scale+bias, fp16 x and y" % M,
+            "linears_per_step": 3,
+            "algorithmic_flops_per_step": r["step_flops"],
+            "percent_of_f16_peak": r["percent_of_f16_peak"],
+            "preheat_ms": r["preheat_ms"],
+            # what the matrix instruction sustains here from registers: alone, and with two or
+            # three packed-fp16 vector instructions per matrix instruction (in-register dequantization)
+            "measured_mfma_tflops": {"alone": round(ctx.probe_mfma_rate(0), 1),
+                                     "with_2_valu": round(ctx.probe_mfma_rate(2), 1),
+                                     "with_3_valu": round(ctx.probe_mfma_rate(3), 1)},
+            "gpu_event_ms_per_step": round(r["gpu_ms"] / args.steps, 5),
+            **device_fields(ctx.info()),
+        },
+        "roofline": r["roofline"],
+    }
+    if "cpu_baseline" in r:
+        result["cpu_baseline"] = r["cpu_baseline"]
     print(json.dumps(result), flush=True)
-    for copy in weights:
-        for weight in copy:
-            weight.destroy()
     return 0
 
 
-def bench_w8a8(engine, ctx, args):
+# ---- W8A8 --------------------------------------------------------------------------------------
+
+def measure_w8a8(engine, ctx, steps, warmup, preheat_ms, with_cpu=True):
     """One step: quantize the activations once, then three projections that share them."""
     M, K, N, count = W8A8["M"], W8A8["K"], W8A8["N"], W8A8["projections"]
     rows = [engine.synth_w8_rows(2000 + i, 0.02, N, K) for i in range(count)]
@@ -287,32 +452,23 @@ def bench_w8a8(engine, ctx, args):
     out_ptr = [ctx.alloc(M * N * 4) for _ in range(count)]
     acc_ptr = [ctx.alloc(M * N * 4) for _ in range(count)]
 
-    def run_steps(steps):
-        for _ in range(steps):
+    def run_steps(n):
+        for _ in range(n):
             ctx.quantize_i8_device(x_ptr, M, K, q_ptr, s_ptr)
             ctx.w8a8_linear_multi_device(weights, q_ptr, s_ptr, M, bias_ptr, out_ptr, acc_ptr)
 
-    wall, gpu_ms, kernel_ms, launches = time_steps(ctx, run_steps, args.steps, args.warmup)
+    timed = time_steps(ctx, run_steps, steps, warmup, preheat_ms, preheat_batch=200)
     step_ops = 2.0 * M * K * N * count
-    value = step_ops * args.steps / wall / 1e12
-    achieved = step_ops * args.steps / (kernel_ms * 1e-3) / 1e12
+    value = step_ops * steps / timed["wall"] / 1e12
+    achieved = step_ops * steps / (timed["kernel_ms"] * 1e-3) / 1e12
+    per_launch = timed["per_launch_us"]
+    gemm_us = float(np.median(per_launch[1::2])) if len(per_launch) == 2 * steps else None
+    weight_bytes = count * N * (4 + K)
     result = {
-        "metric": "w8a8_tops_m64_k1024_n4096",
-        "value": round(value, 3),
-        "unit": "TOP/s",
-        **common_fields(args, wall),
-        "dtype": "i8 x i8, i32 accumulate, f32 epilogue",
-        "data": "synthetic (seeded N(0,0.02) weights absmax-quantized per row, N(0,1) fp32 activations "
-                "quantized per token on the GPU)",
-        "config": {
-            "workload": "per-token int8 quantization then %d projections M=%d K=%d N=%d with bias"
-                        % (count, M, K, N),
-            "launches_per_step": 2,
-            "projections_share_one_launch": True,
-            "algorithmic_ops_per_step": step_ops,
-            "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
-            **device_fields(ctx.info()),
-        },
+        "tops": round(value, 3), "wall": timed["wall"], "gpu_ms": timed["gpu_ms"],
+        "preheat_ms": round(timed["preheat_ms"], 1), "step_ops": step_ops,
+        "projection_launch_us_p50": round(gemm_us, 2) if gemm_us else None,
+        "weight_gb_per_s_at_p50": round(weight_bytes / (gemm_us * 1e-6) / 1e9, 1) if gemm_us else None,
         "roofline": {
             "bound": "mfma",
             "achieved": round(achieved, 3),
@@ -321,13 +477,13 @@ def bench_w8a8(engine, ctx, args):
             "frac": round(achieved / I8_MFMA_PEAK_TOPS, 5),
             "traffic": None,
             "kernel": "w8a8_kernel (quantize_i8_kernel included in the time)",
-            "launches": int(launches),
-            "avg_kernel_us": round(kernel_ms * 1e3 / max(launches, 1), 3),
+            "launches": timed["launches"],
+            "avg_kernel_us": round(timed["kernel_ms"] * 1e3 / max(timed["launches"], 1), 3),
         },
     }
-    if not args.no_cpu:
+    if with_cpu:
         import oracle  # test infrastructure: the timed CPU baseline and the bit-exactness check
-        threads = min(os.cpu_count() or 1, 16)
+        threads, _ = host_threads()
         q_ref, s_ref = oracle.quantize_i8(x)
         repeats, t0 = 20, time.perf_counter()
         for _ in range(repeats):
@@ -339,15 +495,87 @@ def bench_w8a8(engine, ctx, args):
         for i in range(count):
             exact &= bool(np.array_equal(ctx.download(acc_ptr[i], (M, N), np.int32), refs[i][1]))
             exact &= bool(np.array_equal(ctx.download(out_ptr[i], (M, N), np.float32), refs[i][0]))
-        result["config"]["bit_exact_vs_oracle"] = exact
+        result["bit_exact_vs_oracle"] = exact
         result["cpu_baseline"] = {
             "value": round(step_ops / seconds / 1e12, 5), "unit": "TOP/s", "cores": threads, "kind": "port",
             "sample": "%d passes of the same step (mean), oracle restatement of quantize_i8 and "
-                      "matrix_sequence_i8_quantized, OpenMP static over output rows, %.2f ms per pass" % (repeats, seconds * 1e3)}
-    print(json.dumps(result), flush=True)
+                      "matrix_sequence_i8_quantized, OpenMP static over output rows, %.2f ms per pass"
+                      % (repeats, seconds * 1e3)}
+    for pointer in [x_ptr, q_ptr, s_ptr] + bias_ptr + out_ptr + acc_ptr:
+        ctx.free(pointer)
     for weight in weights:
         ctx.w8a8_destroy(weight)
+    return result
+
+
+def bench_w8a8(engine, ctx, args):
+    M, K, N, count = W8A8["M"], W8A8["K"], W8A8["N"], W8A8["projections"]
+    r = measure_w8a8(engine, ctx, args.steps, args.warmup, args.preheat_ms, with_cpu=not args.no_cpu)
+    result = {
+        "metric": "w8a8_tops_m64_k1024_n4096",
+        "value": r["tops"],
+        "unit": "TOP/s",
+        **common_fields(args, r["wall"]),
+        "dtype": "i8 x i8, i32 accumulate, f32 epilogue",
+        "data": "synthetic (seeded N(0,0.02) weights absmax-quantized per row, N(0,1) fp32 activations "
+                "quantized per token on the GPU)",
+        "config": {
+            "workload": "per-token int8 quantization then %d projections M=%d K=%d N=%d with bias"
+                        % (count, M, K, N),
+            "launches_per_step": 2,
+            "projections_share_one_launch": True,
+            "algorithmic_ops_per_step": r["step_ops"],
+            "preheat_ms": r["preheat_ms"],
+            "projection_launch_us_p50": r["projection_launch_us_p50"],
+            "weight_gb_per_s_at_p50": r["weight_gb_per_s_at_p50"],
+            "gpu_event_ms_per_step": round(r["gpu_ms"] / args.steps, 5),
+            **device_fields(ctx.info()),
+        },
+        "roofline": r["roofline"],
+    }
+    if "cpu_baseline" in r:
+        result["config"]["bit_exact_vs_oracle"] = r["bit_exact_vs_oracle"]
+        result["cpu_baseline"] = r["cpu_baseline"]
+    print(json.dumps(result), flush=True)
     return 0
+
+
+# ---- the secondary figures of the default line --------------------------------------------------
+
+def secondary_figures(engine, ctx, work, args):
+    """The other configurations of the headline metric, measured briefly on the same weights."""
+    out = {}
+    for M in (2, 4, 8):
+        r = measure_layer(ctx, work, M, 100, 10, 20.0)
+        out["verify_m%d" % M] = {
+            "gb_per_s": round(r["value"], 1),
+            "percent_of_hbm_peak": round(100.0 * r["value"] / HBM_PEAK_GBPS, 2),
+            "steps": 100, "warmup": 10,
+            "roofline": {"bound": "hbm", "achieved": round(r["achieved"], 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4),
+                         "kernel": "q4_stream_kernel", "avg_kernel_us": round(r["avg_kernel_us"], 3),
+                         "algorithmic_bytes_per_launch": round(r["bytes_per_launch"], 1)},
+            "kernel_us_per_step_p50": round(r["kernel_us_per_step"][1], 2),
+            "kernel_us_per_launch_p50_in_launch_order": r["launch_p50"],
+        }
+    # prefill: the MLP weights of the layer (every copy), M = 512
+    mlp = [[copy[4], copy[5], copy[6]] for copy in work.weights]
+    host = {name: work.host[name] for name, _, _ in PREFILL}
+    p = measure_prefill(engine, ctx, 512, 30, 5, 50.0, weights=mlp, host=host, with_cpu=not args.no_cpu)
+    out["prefill_m512"] = {"tflops": p["tflops"], "percent_of_f16_peak": p["percent_of_f16_peak"],
+                           "steps": 30, "warmup": 5, "linears_per_step": 3,
+                           "algorithmic_flops_per_step": p["step_flops"], "roofline": p["roofline"]}
+    if "cpu_baseline" in p:
+        out["prefill_m512"]["cpu_baseline"] = p["cpu_baseline"]
+    w = measure_w8a8(engine, ctx, 200, 20, 20.0, with_cpu=not args.no_cpu)
+    out["w8a8_m64_k1024_n4096"] = {"tops": w["tops"], "steps": 200, "warmup": 20, "projections_per_step": 3,
+                                   "projection_launch_us_p50": w["projection_launch_us_p50"],
+                                   "weight_gb_per_s_at_p50": w["weight_gb_per_s_at_p50"],
+                                   "roofline": w["roofline"]}
+    if "cpu_baseline" in w:
+        out["w8a8_m64_k1024_n4096"]["bit_exact_vs_oracle"] = w["bit_exact_vs_oracle"]
+        out["w8a8_m64_k1024_n4096"]["cpu_baseline"] = w["cpu_baseline"]
+    return out
 
 
 def main():
@@ -359,6 +587,8 @@ def main():
     parser.add_argument("--rows", type=int, default=None,
                         help="activation rows M (default 1; 512 for --workload prefill)")
     parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "lm_head", "prefill", "w8a8"])
+    parser.add_argument("--preheat-ms", type=float, default=100.0,
+                        help="GPU time of untimed steps before anything is timed (0: none)")
     parser.add_argument("--unfused", action="store_true",
                         help="one launch per linear instead of shared-x launches for q|k|v and gate|up")
     parser.add_argument("--graph", action="store_true",
@@ -366,7 +596,9 @@ def main():
                              "the timed pass; the per-kernel pass stays eager")
     parser.add_argument("--fused-mlp", action="store_true",
                         help="gate|up launch applies silu(gate)*up (one output instead of two)")
-    parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline legs")
+    parser.add_argument("--no-secondary", action="store_true",
+                        help="default workload only: leave out the verify / prefill / W8A8 figures")
     parser.add_argument("--verbose", action="store_true")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -389,79 +621,37 @@ def main():
     copies = {"layer_m1": args.copies, "config1": max(args.copies, 600), "lm_head": 2}[args.workload]
     if args.workload == "lm_head" and args.steps == 400 and args.warmup == 40:
         args.steps, args.warmup = 60, 6
+    headline = args.workload == "layer_m1" and M == 1 and not (args.unfused or args.graph or args.fused_mlp)
+    with_secondary = headline and not args.no_secondary
     ctx = engine.Context(0)  # raises without a GPU
     info = ctx.info()
-    calls, weights, host, x_ptr, y_ptr = build_workload(engine, ctx, shapes, M, copies, meta_kind,
-                                                        args.verbose, fuse=not args.unfused,
-                                                        silu=args.fused_mlp)
-    launches_per_step = len(calls[0])
-    step_bytes = sum(q4_bytes(N, K, M) for _, N, K in shapes)
-
-    def run_steps(count):
-        for step in range(count):
-            ctx.q4_sequence(calls[step % copies])
-
-    graphs = [ctx.q4_sequence_record(c) for c in calls] if args.graph else None
-
-    def run_timed(count):
-        if graphs is None:
-            return run_steps(count)
-        for step in range(count):
-            ctx.graph_launch(graphs[step % copies])
-
-    run_timed(args.warmup)
-    ctx.sync()
-    t0 = time.perf_counter()
-    ctx.timer_begin()
-    run_timed(args.steps)
-    gpu_ms = ctx.timer_end()  # waits for the stream
-    ctx.sync()
-    wall = time.perf_counter() - t0
+    work = LayerWorkload(engine, ctx, shapes, copies, meta_kind, max(M, 8) if with_secondary else M,
+                         args.verbose)
+    r = measure_layer(ctx, work, M, args.steps, args.warmup, args.preheat_ms, fuse=not args.unfused,
+                      silu=args.fused_mlp, graph=args.graph)
+    step_bytes, launches_per_step = r["step_bytes"], r["launches_per_step"]
 
     # the same steps over one copy only: what a cache-resident weight set would show
     hot_steps = min(args.steps, 200)
     for step in range(args.warmup):
-        ctx.q4_sequence(calls[0])
+        ctx.q4_sequence(r["calls"][0])
     ctx.timer_begin()
     for step in range(hot_steps):
-        ctx.q4_sequence(calls[0])
+        ctx.q4_sequence(r["calls"][0])
     hot_ms = ctx.timer_end()
-
-    # second pass of the same steps with an event pair bound to every dispatch
-    ctx.profile_begin()
-    run_steps(args.steps)
-    kernel_ms, launches = ctx.profile_end()
-    per_launch = ctx.profile_durations()
-    # kernel time of each step (its launches, and the slice reductions some of them carry)
-    per_step = per_launch[:len(per_launch) // args.steps * args.steps].reshape(args.steps, -1).sum(axis=1)
-    p10, p50, p90 = (float(np.percentile(per_step, q)) for q in (10, 50, 90))
-    # median duration of each launch of a step, in launch order (only when every launch is one kernel)
-    launch_p50 = None
-    if len(per_launch) == args.steps * launches_per_step:
-        launch_p50 = [round(float(v), 2)
-                      for v in np.median(per_launch.reshape(args.steps, launches_per_step), axis=0)]
 
     # measured plain-read ceiling: whole 2 GiB pass, and launches the size of one weight matrix
     read_long = ctx.probe_read_bandwidth(2 << 30, 3, 1, 0)
     read_short = ctx.probe_read_bandwidth(2 << 30, 3, 1, int(step_bytes / launches_per_step))
 
-    value = step_bytes * args.steps / wall / 1e9
-    bytes_per_launch = step_bytes / launches_per_step
-    avg_kernel_us = kernel_ms * 1e3 / max(launches, 1)
-    achieved = bytes_per_launch / (avg_kernel_us * 1e-6) / 1e9
+    value, p = r["value"], r["kernel_us_per_step"]
     result = {
         "metric": {"layer_m1": "q4_gemv_hbm_gb_per_s_m%d_27b_layer",
                    "config1": "q4_gemv_hbm_gb_per_s_m%d_k1024_n3584",
                    "lm_head": "q4_gemv_hbm_gb_per_s_m%d_lm_head_248320x5120"}[args.workload] % M,
         "value": round(value, 2),
         "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall * 1e3 / args.steps, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
+        **common_fields(args, r["wall"]),
         "dtype": "u4 codes x f16, f32 accumulate",
         "data": "synthetic (seeded N(0,0.02) weights min/max-quantized to affine-Q4 g64, N(0,1) "
                 "fp16 activations)",
@@ -477,44 +667,41 @@ def main():
             "algorithmic_bytes_per_step": step_bytes,
             "weight_copies_rotated": copies,
             "rotated_bytes": step_bytes * copies,
+            "preheat_ms": round(r["preheat_ms"], 1),
             "single_copy_gb_per_s": round(step_bytes * hot_steps / (hot_ms * 1e-3) / 1e9, 1),
             "percent_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-            "gpu_event_ms_per_step": round(gpu_ms / args.steps, 5),
-            "kernel_us_per_step_p10_p50_p90": [round(p10, 2), round(p50, 2), round(p90, 2)],
-            "gb_per_s_at_p50_kernel_time": round(step_bytes / (p50 * 1e-6) / 1e9, 1),
-            "kernel_us_per_launch_p50_in_launch_order": launch_p50,
-            "weights_sha256": weights_digest(host, shapes),
-            "device": info.name.decode(errors="replace").strip(),
-            "arch": info.arch.decode(errors="replace"),
-            "max_clock_mhz": info.clock_mhz, "memory_clock_mhz": info.memory_clock_mhz,
-            "memory_bus_bits": info.memory_bus_bits,
-            "compute_units": info.compute_units,
+            "gpu_event_ms_per_step": round(r["gpu_ms"] / args.steps, 5),
+            "kernel_us_per_step_p10_p50_p90": [round(p[0], 2), round(p[1], 2), round(p[2], 2)],
+            "gb_per_s_at_p50_kernel_time": round(step_bytes / (p[1] * 1e-6) / 1e9, 1),
+            "kernel_us_per_launch_p50_in_launch_order": r["launch_p50"],
+            "weights_sha256": work.digest(),
+            **device_fields(info),
             "measured_read_gb_per_s": {"one_2GiB_pass": round(read_long, 1),
                                        "matrix_sized_launches": round(read_short, 1)},
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(achieved, 2),
+            "achieved": round(r["achieved"], 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": round(bytes_per_launch * MEASURED_TRAFFIC_RATIO_LAYER_M1)
-                       if args.workload == "layer_m1" and M == 1 and not args.unfused else None,
+            "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4),
+            "traffic": round(r["bytes_per_launch"] * MEASURED_TRAFFIC_RATIO_LAYER_M1) if headline else None,
+            "traffic_source": ("rocprofv3 FETCH_SIZE + WRITE_SIZE per algorithmic byte = %.3f, read from "
+                               "profiles/q4_stream_kernel_layer_m1.md (not measured in this run)"
+                               % MEASURED_TRAFFIC_RATIO_LAYER_M1) if headline else None,
             "kernel": "q4_stream_kernel",
-            "launches": int(launches),
-            "avg_kernel_us": round(avg_kernel_us, 3),
-            "algorithmic_bytes_per_launch": round(bytes_per_launch, 1),
+            "launches": r["launches"],
+            "avg_kernel_us": round(r["avg_kernel_us"], 3),
+            "algorithmic_bytes_per_launch": round(r["bytes_per_launch"], 1),
         },
     }
     if not args.no_cpu:
         import oracle  # test infrastructure, used here only as the timed CPU baseline
-        result["cpu_baseline"] = cpu_baseline(oracle, shapes, host, M, meta_kind)
+        result["cpu_baseline"] = cpu_baseline_layer(oracle, shapes, work.host, M, meta_kind)
+    if with_secondary:
+        result["secondary"] = secondary_figures(engine, ctx, work, args)
     print(json.dumps(result), flush=True)
-    for graph in graphs or []:
-        ctx.graph_destroy(graph)
-    for copy in weights:
-        for weight in copy:
-            weight.destroy()
+    work.destroy()
     ctx.close()
     return 0
 

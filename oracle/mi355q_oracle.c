@@ -587,3 +587,48 @@ void orc_recipe_qwen38_weights(uint32_t seed, size_t group_count, uint8_t *quant
     }
 }
 
+/* Host read bandwidth in the manner of the reference's target probe (read_worker /
+ * run_read_benchmark, tools/target_probe.c:60-160): every thread sums its own share of a
+ * buffer of 64-bit words with four independent accumulators, pass after pass, until
+ * `seconds` have gone by; the figure is bytes read / the longest thread's time, in GiB/s.
+ * The buffer (bytes, at least 64 MiB to get past the caches) is written once first.
+ * Not part of the path: context for the cpu_baseline figures.  Returns 0 on failure. */
+double orc_probe_read_gib_per_s(size_t bytes, int threads, double seconds, uint64_t *checksum_out)
+{
+    const size_t words = bytes / sizeof(uint64_t);
+    if (threads < 1 || words < (size_t)threads * 4u) return 0.0;
+    uint64_t *buffer = (uint64_t *)malloc(words * sizeof(uint64_t));
+    if (buffer == NULL) return 0.0;
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (size_t i = 0; i < words; ++i) buffer[i] = (uint64_t)i * 0x9e3779b97f4a7c15ull;
+    uint64_t total_bytes = 0, checksum = 0;
+    double longest = 0.0;
+#pragma omp parallel num_threads(threads) reduction(+ : total_bytes) reduction(^ : checksum) reduction(max : longest)
+    {
+        const int index = omp_get_thread_num(), count = omp_get_num_threads();
+        const size_t share = words / (size_t)count;
+        const uint64_t *data = buffer + (size_t)index * share;
+        const size_t mine = (index == count - 1 ? words - (size_t)index * share : share) & ~(size_t)3;
+        uint64_t sum0 = 0, sum1 = 0, sum2 = 0, sum3 = 0, read = 0;
+#pragma omp barrier
+        const double start = omp_get_wtime();
+        double now;
+        do {
+            for (size_t i = 0; i < mine; i += 4) {
+                sum0 += data[i];
+                sum1 += data[i + 1];
+                sum2 += data[i + 2];
+                sum3 += data[i + 3];
+            }
+            read += (uint64_t)mine * sizeof(uint64_t);
+            now = omp_get_wtime();
+        } while (now - start < seconds);
+        total_bytes += read;
+        checksum ^= sum0 ^ sum1 ^ sum2 ^ sum3;
+        longest = now - start;
+    }
+    free(buffer);
+    if (checksum_out) *checksum_out = checksum;
+    return longest > 0.0 ? (double)total_bytes / longest / 1073741824.0 : 0.0;
+}
+

@@ -145,6 +145,10 @@ void orc_q8_weight_quantize(const float *w, uint32_t N, uint32_t K,
 void orc_recipe_qwen38_weights(uint32_t seed, size_t group_count, uint8_t *quants,
                                uint16_t *meta_interleaved);
 
+/* Host read bandwidth, GiB/s, in the manner of tools/target_probe.c:60-160 (threads summing
+ * their shares of a buffer for `seconds`); context for the CPU baseline, not part of the path. */
+double orc_probe_read_gib_per_s(size_t bytes, int threads, double seconds, uint64_t *checksum_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,8 @@ def lib() -> ctypes.CDLL:
         l.orc_q8_weight_quantize.argtypes = [_vp, _u32, _u32, _vp]
         l.orc_recipe_qwen38_weights.restype = None
         l.orc_recipe_qwen38_weights.argtypes = [_u32, _sz, _vp, _vp]
+        l.orc_probe_read_gib_per_s.restype = _c.c_double
+        l.orc_probe_read_gib_per_s.argtypes = [_sz, _int, _c.c_double, _vp]
         _libs["oracle"] = l
     return _libs["oracle"]
 
@@ -253,3 +255,9 @@ def q8_weight_quantize(w):
     rows = np.empty(N * (4 + K), dtype=np.uint8)
     lib().orc_q8_weight_quantize(_p(w), N, K, _p(rows))
     return rows
+
+
+def probe_read_gib_per_s(nbytes=256 << 20, threads=1, seconds=0.5):
+    """Host read bandwidth (GiB/s) at `threads` threads, the reference's target-probe measurement."""
+    return lib().orc_probe_read_gib_per_s(nbytes, threads, seconds, None)
+
