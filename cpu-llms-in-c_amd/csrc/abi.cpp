@@ -69,6 +69,11 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->trace = set && strcmp(value, "0") != 0;
         return MI355Q_OK;
     }
+    if (strcmp(name, "w8a8") == 0) {  // "1" .. "4": tiles per workgroup of the W8A8 kernel, whatever the tile count
+        if (set && (strlen(value) != 1 || value[0] < '1' || value[0] > '4')) return MI355Q_ERROR_INVALID;
+        ctx->w8a8_tiles = set ? value[0] - '0' : 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "in_kernel_slices") == 0) {  // "0": a second kernel adds the K slices
         ctx->columns_share_xcd = ctx->columns_probed && !(set && strcmp(value, "0") == 0);
         return MI355Q_OK;

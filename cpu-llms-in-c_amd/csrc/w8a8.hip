@@ -134,14 +134,14 @@ causal_q8_windows_kernel(const float *__restrict__ input, const float *__restric
 
 constexpr uint32_t kW8a8Targets = 4;
 // Up to four weights of the same K against one quantized activation: workgroup ranges map to
-// weights (first_tile), one launch.
+// weights (first_group), one launch.
 struct W8a8Params {
     const uint4 *tiles[kW8a8Targets];
     const float *wscales[kW8a8Targets];
     const float *bias[kW8a8Targets];  // [N] or null
     float *out[kW8a8Targets];         // [M][N]
     int32_t *acc[kW8a8Targets];       // [M][N] or null
-    uint32_t N[kW8a8Targets], first_tile[kW8a8Targets];
+    uint32_t N[kW8a8Targets];
     uint32_t targets;
     const int8_t *q;       // [M][K]
     const float *xscales;  // [M]
@@ -149,17 +149,22 @@ struct W8a8Params {
     // 0: out[m][n] = ((float)acc * wscale) * xscale + bias (matrix_i8_rows);
     // 1: out[n][m] = bias + (wscale * xscale) * (float)acc (stream_conv_cells, minimindo_mimi.c:869-880)
     int channel_major;
+    // workgroups [first_group[t], first_group[t+1]) work on weight t, each on the kernel's TPW
+    // consecutive tiles of it
+    uint32_t first_group[kW8a8Targets];
 };
 
-// A workgroup of four waves owns one tile of 16 weight rows and MB*16 activation
-// rows; the waves split the 64-column steps (wave w: steps w, w+4, ...) and add
-// their int32 partial sums through LDS.  A wave fetches four of its steps (weights and
-// activations) before the first matrix instruction: at K = 1024 that is all of them, one
-// round trip to memory instead of four.
-template <int MB>
+// A workgroup of four waves owns TPW consecutive tiles of 16 weight rows of one weight and
+// MB*16 activation rows; the waves split the 64-column steps (wave w: steps w, w+4, ...) and
+// add their int32 partial sums through LDS.  A wave fetches four of its steps (activations,
+// and the weights of all its tiles) before the first matrix instruction: at K = 1024 that is
+// all of them, one round trip to memory instead of four.  The activation fragments stay in
+// registers across the workgroup's tiles.  The scales and the bias an output thread needs are
+// fetched at the start of the kernel, so their latency is not in the epilogue.
+template <int MB, int TPW>
 __global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
 {
-    __shared__ int red[4][MB][4][64];
+    __shared__ int red[4][TPW][MB][4][64];
     constexpr int AHEAD = 4;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -167,72 +172,123 @@ __global__ void __launch_bounds__(256) w8a8_kernel(const W8a8Params p)
     uint32_t target = 0;
 #pragma unroll
     for (uint32_t t = 1; t < kW8a8Targets; ++t)
-        if (t < p.targets && blockIdx.x >= p.first_tile[t]) target = t;
-    const uint32_t tile = blockIdx.x - p.first_tile[target];
+        if (t < p.targets && blockIdx.x >= p.first_group[t]) target = t;
+    const uint32_t N = p.N[target], NT = (N + 15u) / 16u;
+    const uint32_t tile0 = (blockIdx.x - p.first_group[target]) * TPW;
     const uint32_t m0 = blockIdx.y * (MB * 16u);
-    const uint32_t N = p.N[target];
 
-    intx4 acc[MB];
+    // what this thread's outputs need: it writes, for every tile t and fragment i, the element
+    // (row m0 + 16 i + 4 (lane / 16) + wave, column 16 (tile0 + t) + lane % 16)
+    float my_wscale[TPW], my_bias[TPW], my_xscale[MB];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) acc[i] = intx4{0, 0, 0, 0};
-    const uint4 *tile_words = p.tiles[target] + (size_t)tile * p.KS * 64u + lane;
+    for (int t = 0; t < TPW; ++t) {
+        const uint32_t n = (tile0 + t) * 16u + r;
+        my_wscale[t] = n < N ? p.wscales[target][n] : 0.0f;
+        my_bias[t] = n < N && p.bias[target] ? p.bias[target][n] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+        const uint32_t m = m0 + 16u * i + 4u * kq + wave;
+        my_xscale[i] = m < p.M ? p.xscales[m] : 0.0f;
+    }
+
+    intx4 acc[TPW][MB];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int i = 0; i < MB; ++i) acc[t][i] = intx4{0, 0, 0, 0};
+    const uint4 *tile_words[TPW];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        const uint32_t tile = tile0 + t < NT ? tile0 + t : NT - 1u;  // a group's last tiles may not exist
+        tile_words[t] = p.tiles[target] + (size_t)tile * p.KS * 64u + lane;
+    }
+    // Every load below is unconditional (a load under a per-lane condition ends a wave's run of
+    // loads in flight): rows past M repeat the last row (never stored), steps past the last
+    // repeat it (their weights are replaced by zeros before the matrix instructions), and
+    // columns past K read the row's last sixteen codes against the tile's zero padding.
     const int8_t *q_rows[MB];
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
-        const uint32_t m = m0 + 16u * i + r;
-        q_rows[i] = m < p.M ? p.q + (size_t)m * p.K : nullptr;
+        uint32_t m = m0 + 16u * i + r;
+        m = m < p.M ? m : p.M - 1u;
+        q_rows[i] = p.q + (size_t)m * p.K;
     }
     for (uint32_t first = wave; first < p.KS; first += 4u * AHEAD) {
-        uint4 b[AHEAD], a[AHEAD][MB];
+        uint4 b[TPW][AHEAD], a[AHEAD][MB];
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) {
-            const uint32_t ks = first + 4u * u;
-            const uint32_t k = ks * 64u + kq * 16u;
-            b[u] = make_uint4(0u, 0u, 0u, 0u);
-            if (ks < p.KS) b[u] = tile_words[(size_t)ks * 64u];
+            uint32_t ks = first + 4u * u;
+            ks = ks < p.KS ? ks : p.KS - 1u;
+            uint32_t k = ks * 64u + kq * 16u;
+            k = k + 16u <= p.K ? k : p.K - 16u;
 #pragma unroll
-            for (int i = 0; i < MB; ++i) {
-                a[u][i] = make_uint4(0u, 0u, 0u, 0u);
-                if (ks < p.KS && q_rows[i] != nullptr && k < p.K) a[u][i] = *(const uint4 *)(q_rows[i] + k);
-            }
+            for (int t = 0; t < TPW; ++t) b[t][u] = load_stream(tile_words[t] + (size_t)ks * 64u);
+#pragma unroll
+            for (int i = 0; i < MB; ++i) a[u][i] = *(const uint4 *)(q_rows[i] + k);
         }
 #pragma unroll
-        for (int u = 0; u < AHEAD; ++u)
+        for (int u = 1; u < AHEAD; ++u)
+            if (first + 4u * u >= p.KS) {  // uniform: no such step
 #pragma unroll
-            for (int i = 0; i < MB; ++i)
-                acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a[u][i]),
-                                                               __builtin_bit_cast(intx4, b[u]), acc[i], 0, 0, 0);
+                for (int t = 0; t < TPW; ++t) b[t][u] = make_uint4(0u, 0u, 0u, 0u);
+            }
+#pragma unroll
+        for (int t = 0; t < TPW; ++t)
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    acc[t][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a[u][i]),
+                                                                      __builtin_bit_cast(intx4, b[t][u]),
+                                                                      acc[t][i], 0, 0, 0);
     }
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int t = 0; t < TPW; ++t)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) red[wave][i][j][lane] = acc[i][j];
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) red[wave][t][i][j][lane] = acc[t][i][j];
     __syncthreads();
-    // lane (r, kq) of fragment i holds activation rows 16*i + 4*kq + j, weight row 16*tile + r
-    const float *wscales = p.wscales[target], *bias = p.bias[target];
+    // lane (r, kq) of fragment i holds activation rows 16*i + 4*kq + j, weight row 16*tile + r;
+    // thread (wave, lane) finishes the elements j = wave of its lane
     float *out = p.out[target];
     int32_t *acc_out = p.acc[target];
-    for (uint32_t e = threadIdx.x; e < MB * 4u * 64u; e += 256u) {
-        const uint32_t l = e & 63u, j = (e >> 6) & 3u, i = e >> 8;
-        const int sum = red[0][i][j][l] + red[1][i][j][l] + red[2][i][j][l] + red[3][i][j][l];
-        const uint32_t m = m0 + 16u * i + 4u * (l >> 4) + j;
-        const uint32_t n = tile * 16u + (l & 15u);
-        if (m >= p.M || n >= N) continue;
-        const size_t at = (size_t)m * N + n;
-        if (acc_out) acc_out[at] = sum;
-        {
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+            const int sum = red[0][t][i][wave][lane] + red[1][t][i][wave][lane] + red[2][t][i][wave][lane] +
+                            red[3][t][i][wave][lane];
+            const uint32_t m = m0 + 16u * i + 4u * kq + wave;
+            const uint32_t n = (tile0 + t) * 16u + r;
+            if (tile0 + t >= NT || m >= p.M || n >= N) continue;
+            const size_t at = (size_t)m * N + n;
+            if (acc_out) acc_out[at] = sum;
+            {
 #pragma clang fp contract(off)
-            if (p.channel_major) {
-                float value = wscales[n] * p.xscales[m];
-                value = value * (float)sum;
-                out[(size_t)n * p.M + m] = (bias ? bias[n] : 0.0f) + value;
-            } else {
-                float value = (float)sum * wscales[n];
-                value = value * p.xscales[m];
-                value = value + (bias ? bias[n] : 0.0f);
-                out[at] = value;
+                if (p.channel_major) {
+                    float value = my_wscale[t] * my_xscale[i];
+                    value = value * (float)sum;
+                    out[(size_t)n * p.M + m] = my_bias[t] + value;
+                } else {
+                    float value = (float)sum * my_wscale[t];
+                    value = value * my_xscale[i];
+                    value = value + my_bias[t];
+                    out[at] = value;
+                }
             }
         }
+}
+
+template <int MB>
+static hipError_t launch_w8a8(mi355q_context *ctx, dim3 grid, uint32_t tiles_per_group, const W8a8Params &p)
+{
+    switch (tiles_per_group) {
+    case 1: return launch(ctx, w8a8_kernel<MB, 1>, grid, dim3(256), 0, p);
+    case 2: return launch(ctx, w8a8_kernel<MB, 2>, grid, dim3(256), 0, p);
+    case 3: return launch(ctx, w8a8_kernel<MB, 3>, grid, dim3(256), 0, p);
+    default: return launch(ctx, w8a8_kernel<MB, 4>, grid, dim3(256), 0, p);
     }
 }
 
@@ -458,7 +514,6 @@ int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targ
         p.out[t] = targets[t].out;
         p.acc[t] = targets[t].acc;
         p.N[t] = weight->N;
-        p.first_tile[t] = tiles;
         tiles += weight->NT;
         bias_bytes += (size_t)weight->N * 4u;
         out_bytes += (size_t)M * weight->N * 4u * (targets[t].acc ? 2u : 1u);
@@ -492,13 +547,25 @@ int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targ
             }
         }
     }
+    // Tiles per workgroup (they share the workgroup's activation registers).  Measured at
+    // M = 64, K = 1024, three weights of 4096 rows (768 tiles): 10.0 / 10.0 / 11.6 / 10.1 us for
+    // 1 / 2 / 3 / 4 tiles, so a launch takes one unless the option "w8a8" says otherwise.
+    const uint32_t m_blocks = M > 32u ? (M + 63u) / 64u : 1u;
+    uint32_t per_group = ctx->w8a8_tiles ? (uint32_t)ctx->w8a8_tiles : 1u;
+    per_group = per_group < 1u ? 1u : per_group > 4u ? 4u : per_group;
+    uint32_t groups = 0;
+    for (uint32_t t = 0; t < count; ++t) {
+        p.first_group[t] = groups;
+        groups += (targets[t].weight->NT + per_group - 1u) / per_group;
+    }
+    const dim3 grid(groups, m_blocks);
     hipError_t launched;
     if (M > 32u)
-        launched = launch(ctx, w8a8_kernel<4>, dim3(tiles, (M + 63u) / 64u), dim3(256), 0, p);
+        launched = launch_w8a8<4>(ctx, grid, per_group, p);
     else if (M > 16u)
-        launched = launch(ctx, w8a8_kernel<2>, dim3(tiles, 1), dim3(256), 0, p);
+        launched = launch_w8a8<2>(ctx, grid, per_group, p);
     else
-        launched = launch(ctx, w8a8_kernel<1>, dim3(tiles, 1), dim3(256), 0, p);
+        launched = launch_w8a8<1>(ctx, grid, per_group, p);
     if (launched != hipSuccess) return fail_hip(launched, "w8a8 kernel launch", error, error_capacity);
     if (!device) {
         for (uint32_t t = 0; t < count; ++t) {

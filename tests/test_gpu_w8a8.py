@@ -34,9 +34,33 @@ def test_config5(engine, oracle, gpu):
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 16, 16), (3, 48, 20), (17, 560, 100), (40, 512, 2048),
-                                   (130, 2048, 512), (64, 1024, 4100)])
+                                   (130, 2048, 512), (64, 1024, 4100), (5, 1024, 40), (17, 3072, 1000),
+                                   (33, 1024, 16400), (64, 2048, 12304)])
 def test_shapes(engine, oracle, gpu, M, K, N):
+    """A workgroup takes one to four tiles by the launch's tile count (3, 63, 1025 and 769 tiles
+    among these), its last tiles may not exist, K of one to three 1024-column rounds and ragged
+    ones, row counts that end inside a fragment."""
     check(engine, oracle, gpu, M, K, N, 7 + M, bias=(M % 2 == 0))
+
+
+@pytest.mark.parametrize("M,K,N,channel_major", [(64, 1024, 4096, False), (21, 2048, 530, True)])
+def test_both_kernels_give_the_same_bits(engine, gpu, force, M, K, N, channel_major):
+    """Several tiles per workgroup and one tile per workgroup on the same call."""
+    x = engine.synth_normal_f32(5, 1.0, M * K).reshape(M, K)
+    rows = engine.synth_w8_rows(6, 0.02, N, K)
+    bias = engine.synth_normal_f32(7, 1.0, N)
+    q, scales = gpu.quantize_i8(x)
+    weight = gpu.w8a8_prepare(rows, N, K)
+    try:
+        print(f"w8a8 both kernels M={M} K={K} N={N} channel_major={channel_major}", flush=True)
+        shared = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
+        force("w8a8", "1")
+        per_tile = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
+    finally:
+        gpu.w8a8_destroy(weight)
+    assert shared[1].tobytes() == per_tile[1].tobytes()
+    assert np.array_equal(shared[0].view(np.uint32), per_tile[0].view(np.uint32))
+    assert np.any(shared[1] != 0)
 
 
 def test_reference_golden_vectors(engine, gpu):
