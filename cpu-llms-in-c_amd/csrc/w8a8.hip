@@ -504,7 +504,6 @@ int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targ
     p.KS = targets[0].weight->KS;
     p.targets = count;
     p.channel_major = (flags & MI355Q_W8A8_CHANNEL_MAJOR) != 0;
-    uint32_t tiles = 0;
     size_t bias_bytes = 0, out_bytes = 0;
     for (uint32_t t = 0; t < count; ++t) {
         const mi355q_w8a8_weight *weight = targets[t].weight;
@@ -514,7 +513,7 @@ int mi355q_w8a8_linear_multi(mi355q_context *ctx, const mi355q_w8a8_target *targ
         p.out[t] = targets[t].out;
         p.acc[t] = targets[t].acc;
         p.N[t] = weight->N;
-        tiles += weight->NT;
+
         bias_bytes += (size_t)weight->N * 4u;
         out_bytes += (size_t)M * weight->N * 4u * (targets[t].acc ? 2u : 1u);
     }
