@@ -112,9 +112,9 @@ def host_fields(oracle, threads, allowed):
         "host_cpus_online": os.cpu_count(),
         "host_cpus_allowed": allowed,
         "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
-        "host_read_gib_per_s": {"threads_1": round(oracle.probe_read_gib_per_s(threads=1, seconds=0.4), 2),
-                                "threads_%d" % threads: round(oracle.probe_read_gib_per_s(threads=threads,
-                                                                                         seconds=0.4), 2)},
+        # a 2 GiB buffer: far beyond the last-level caches of any host
+        "host_read_gib_per_s": {"threads_1": round(oracle.probe_read_gib_per_s(2 << 30, 1, 0.5), 2),
+                                "threads_%d" % threads: round(oracle.probe_read_gib_per_s(2 << 30, threads, 0.5), 2)},
     }
 
 
