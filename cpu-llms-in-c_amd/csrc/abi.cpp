@@ -74,6 +74,11 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->w8a8_tiles = set ? value[0] - '0' : 0;
         return MI355Q_OK;
     }
+    if (strcmp(name, "gemm_loads") == 0) {  // "plain": GEMM variant 7 with ordinary weight loads (a cross-check)
+        if (set && strcmp(value, "plain") != 0) return MI355Q_ERROR_INVALID;
+        ctx->gemm_plain_loads = set;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "in_kernel_slices") == 0) {  // "0": a second kernel adds the K slices
         ctx->columns_share_xcd = ctx->columns_probed && !(set && strcmp(value, "0") == 0);
         return MI355Q_OK;

@@ -474,7 +474,11 @@ __device__ __forceinline__ void load_x2(u32x2 &to, uint32_t lane_offset, const c
     asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(to) : "v"(lane_offset), "s"(base) : "memory");
 }
 
-template <int BM, int NTW, bool XT>
+// PLAIN: the weight loads are ordinary loads, whose waits the compiler places itself, instead
+// of asm statements under the kernel's own counted waits.  Slower, and the reference point for
+// the hand-scheduled form: both must give the same bits (a test compares them), which would
+// show a wait that no longer covers its loads after a change of compiler or of the schedule.
+template <int BM, int NTW, bool XT, bool PLAIN = false>
 __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p)
 {
     extern __shared__ uint4 a_lds_raw[];  // [buffer][row][slot], slot = octet ^ (row % 16)
@@ -548,6 +552,11 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         if constexpr (load < AJ) {
             const uint32_t lds_base = lds_wave + buffer * (uint32_t)(BM * 16u * sizeof(uint4));
             load_to_lds<(load - AJ / 2) * 1024>(a_offset[load], x_next, lds_base);
+        } else if constexpr (PLAIN) {
+            if constexpr ((load - AJ) % 2 == 0)
+                codes[(load - AJ) / 2] = *(const u32x4 *)(codes_next + codes_offset[(load - AJ) / 2]);
+            else
+                meta[(load - AJ) / 2] = *(const u32x2 *)(meta_next + meta_offset[(load - AJ) / 2]);
         } else if constexpr ((load - AJ) % 2 == 0) {
             load_x4(codes[(load - AJ) / 2], codes_offset[(load - AJ) / 2], codes_next);
         } else {
@@ -817,6 +826,20 @@ static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &
     return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT>, grid, dim3(256), bytes, p);
 }
 
+// The 17-tile shape with compiler-managed weight loads (option "gemm_loads" = "plain").
+static hipError_t launch_pipe_plain(mi355q_context *ctx, dim3 grid, const GemmParams &p)
+{
+    constexpr size_t bytes = pipe_lds_bytes(128);
+    constexpr int slot = 15;
+    if (!ctx->lds_raised[slot]) {
+        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, 4, true, true>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (status != hipSuccess) return status;
+        ctx->lds_raised[slot] = true;
+    }
+    return launch(ctx, q4_gemm_pipe_kernel<128, 4, true, true>, grid, dim3(256), bytes, p);
+}
+
 int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
                    size_t error_capacity)
 {
@@ -960,7 +983,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     case 4: launched = launch(ctx, q4_gemm_kernel<64, 2, false>, grid, dim3(256), 0, p); break;
     case 5: launched = launch(ctx, q4_gemm_kernel<64, 2, true>, grid, dim3(256), 0, p); break;
     case 6: launched = launch_pipe<4, false>(ctx, grid, p); break;
-    case 7: launched = launch_pipe<4, true>(ctx, grid, p); break;
+    case 7: launched = ctx->gemm_plain_loads ? launch_pipe_plain(ctx, grid, p) : launch_pipe<4, true>(ctx, grid, p); break;
     default: launched = launch_pipe<5, false>(ctx, grid, p); break;
     }
     if (launched != hipSuccess)

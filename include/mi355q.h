@@ -123,6 +123,9 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *   "trace"     = "1"                           prints every launch's decomposition to stderr
  *   "in_kernel_slices" = "0"                    K slices are added by a second kernel
  *   "w8a8"      = "1" .. "4"                    W8A8: weight tiles per workgroup
+ *   "gemm_loads" = "plain"                      GEMM variant 7 built with ordinary weight loads
+ *                                               (compiler-placed waits): the cross-check of the
+ *                                               hand-scheduled kernel, same bits, slower
  * Unknown names and malformed values: status 2. */
 int mi355q_context_set_option(mi355q_context *ctx, const char *name, const char *value,
                               char *error, size_t error_capacity);

@@ -175,3 +175,25 @@ def test_pipelined_kernel_output_alignment(engine, gpu, forced, y_dtype, width, 
         gpu.free(x_ptr)
         gpu.free(y_ptr)
         weight.destroy()
+
+
+@pytest.mark.parametrize("N,K,M,splits", [(17408, 5120, 512, 1), (1104, 2176, 150, 2), (560, 384, 70, 1)])
+def test_hand_scheduled_loads_match_compiler_managed_loads(engine, gpu, force, N, K, M, splits):
+    """The pipelined kernel issues its weight loads as asm statements and waits for them with its
+    own counted s_waitcnt; a second build of the same kernel (the 17-tile shape) uses ordinary loads
+    whose waits the compiler places.  Same bits, or a wait no longer covers its loads."""
+    kind = engine.META_BF16_PLANES
+    quants, meta_a, meta_b = engine.synth_q4_affine(61, 0.02, N, K, kind)
+    x = make_x(engine, 62, M, K).astype(np.float16)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, kind)
+    try:
+        force("q4_gemm", f"7,{splits}")
+        print(f"gemm load forms N={N} K={K} M={M} splits={splits}", flush=True)
+        scheduled = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+        force("gemm_loads", "plain")
+        plain = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+    finally:
+        weight.destroy()
+    assert np.array_equal(scheduled.view(np.uint32), plain.view(np.uint32))
+    assert np.any(scheduled != 0)
+
