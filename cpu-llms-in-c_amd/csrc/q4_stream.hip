@@ -839,6 +839,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.rows = rows;
     p.slice_steps = shape.slice_steps;
     p.slices = shape.slices;
+    uint32_t counted_columns = 0;  // workgroup columns that count arrivals in this launch
     if (p.slices > 1u) {
         for (uint32_t t = 0; t < a.count; ++t) {
             p.n_first[t] = p.n_total;
@@ -847,6 +848,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         const size_t partial_bytes = (size_t)p.slices * a.M * p.n_total * sizeof(float);
         // grid.x of the launch: the workgroup columns that count arrivals
         const uint32_t columns = a.fuse_silu ? (p.NT[0] + shape.tb / 2 - 1) / (shape.tb / 2) : block;
+        counted_columns = columns;
         if (a.no_alloc) {
             if (partial_bytes > kScratchPartialBytes) {
                 set_error(error, error_capacity, "non-allocating call: %zu bytes of slice partial sums "
@@ -903,8 +905,14 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         (void)hipGetLastError();
         return MI355Q_ERROR_INVALID;
     }
-    if (launched != hipSuccess)
+    if (launched != hipSuccess) {
+        // a launch that failed has counted nothing, but the counters of the context must be zero
+        // before the next sliced launch whatever happened here: put them back (not while a graph
+        // is being recorded: a memset node has no place in one)
+        if (p.arrivals != nullptr && !ctx->capturing)
+            (void)hipMemsetAsync(p.arrivals, 0, (size_t)(counted_columns + 8u) * sizeof(uint32_t), ctx->stream);
         return fail_hip(launched, "q4 stream kernel launch", error, error_capacity);
+    }
     if (p.slices > 1u && p.arrivals == nullptr) {
         launched = launch(ctx, q4_stream_reduce_kernel, dim3((p.n_total + 255u) / 256u, a.M), dim3(256), 0, p);
         if (launched != hipSuccess)
