@@ -841,6 +841,43 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         }
         return;
     }
+    // The fp32 partial sums of a K split leave the same way, in two halves of 64 rows (a whole
+    // block of them is a few KB more than the stage): 16 bytes per lane, a row of the block
+    // contiguous, instead of 16-byte pieces of 16 rows 4 N bytes apart.
+    constexpr uint32_t PITCH32 = WIDTH * 4u + 16u;
+    static_assert(PITCH32 % 16u == 0u && (PITCH32 / 16u) % 2u == 1u, "rows start 16-byte aligned, an odd number of 16-byte units apart");
+    static_assert((size_t)(BM / 2) * PITCH32 <= pipe_lds_bytes(BM), "half a block fits the activation stage");
+    const bool partials_through_lds = mode == 3 && p.splits > 1u && p.wide_stores && n_first + WIDTH <= p.N && m0 + BM <= p.M;
+    if (partials_through_lds) {
+        char *const stage = (char *)a_lds_raw;
+        float *const out = p.partials + ((size_t)split * p.M + m0) * p.N + n_first;
+        constexpr uint32_t PIECES = WIDTH / 4u;  // 16-byte pieces per row
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            __syncthreads();  // the stage is free: the main loop's reads, or the first half's
+#pragma unroll
+            for (int t = 0; t < NTW; ++t)
+#pragma unroll
+                for (int i = 0; i < MI / 2; ++i)
+                    *(floatx4 *)(stage + (16u * i + r) * PITCH32 + ((wave * NTW + t) * kTileRows + 4u * kq) * 4u) =
+                        acc[half * (MI / 2) + i][t];
+            if (XT) {
+                if (wave / 2u == (uint32_t)half) {  // this wave's row groups of the shared tile lie in this half
+#pragma unroll
+                    for (int i = 0; i < XI; ++i)
+                        *(floatx4 *)(stage + (16u * (XI * (wave % 2u) + i) + r) * PITCH32 +
+                                     (4u * NTW * kTileRows + 4u * kq) * 4u) = acc_shared[i];
+                }
+            }
+            __syncthreads();
+            for (uint32_t piece = threadIdx.x; piece < BM / 2u * PIECES; piece += 256u) {
+                const uint32_t row = piece / PIECES, column = piece % PIECES * 4u;
+                *(floatx4 *)(out + (size_t)(half * (BM / 2) + row) * p.N + column) =
+                    *(const floatx4 *)(stage + row * PITCH32 + column * 4u);
+            }
+        }
+        return;
+    }
     switch (mode) {
     case 0: store_all(std::integral_constant<int, 0>()); break;
     case 1: store_all(std::integral_constant<int, 1>()); break;
@@ -849,12 +886,40 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     }
 }
 
-// Adds the K splits in split order (a fixed order) and applies the epilogue.
+// Adds the K splits in split order (a fixed order) and applies the epilogue.  WIDE: a thread
+// takes four adjacent outputs of one row (N a multiple of 4, y 16-byte aligned): 16-byte loads
+// of each split's partial sums and one store; the additions are the same, in the same order.
+template <bool WIDE>
 __global__ void __launch_bounds__(256) q4_gemm_reduce_kernel(const GemmParams p)
 {
     const size_t total = (size_t)p.M * p.N;
-    const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    constexpr size_t PER = WIDE ? 4 : 1;
+    const size_t at = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * PER;
     if (at >= total) return;
+    if constexpr (WIDE) {
+        floatx4 value = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t s = 0; s < p.splits; ++s) {
+            const floatx4 more = *(const floatx4 *)(p.partials + (size_t)s * total + at);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) value[j] += more[j];
+        }
+        if (p.residual) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                value[j] += load_as_float(p.residual, p.residual_dtype, p.residual_is_bias ? (at + j) % p.N : at + j);
+        }
+        if (p.y_dtype == MI355Q_F32) {
+            *(floatx4 *)((float *)p.y + at) = value;
+        } else if (p.y_dtype == MI355Q_F16) {
+            typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+            const half4v packed = {(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
+            *(half4v *)((_Float16 *)p.y + at) = packed;
+        } else {
+            *(uint2 *)((uint16_t *)p.y + at) = make_uint2(bf16_bits(value[0]) | (bf16_bits(value[1]) << 16),
+                                                          bf16_bits(value[2]) | (bf16_bits(value[3]) << 16));
+        }
+        return;
+    }
     float value = 0.0f;
     for (uint32_t s = 0; s < p.splits; ++s) value += p.partials[(size_t)s * total + at];
     if (p.residual)
@@ -1057,8 +1122,12 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);
     if (p.splits > 1u) {
         const size_t total = (size_t)a.M * w.N;
-        launched = launch(ctx, q4_gemm_reduce_kernel, dim3((uint32_t)((total + 255u) / 256u)),
-                          dim3(256), 0, p);
+        if (p.wide_stores)
+            launched = launch(ctx, q4_gemm_reduce_kernel<true>, dim3((uint32_t)((total / 4u + 255u) / 256u)),
+                              dim3(256), 0, p);
+        else
+            launched = launch(ctx, q4_gemm_reduce_kernel<false>, dim3((uint32_t)((total + 255u) / 256u)),
+                              dim3(256), 0, p);
         if (launched != hipSuccess)
             return fail_hip(launched, "q4 gemm reduce launch", error, error_capacity);
     }
