@@ -736,35 +736,44 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
                 b_codes[cur], b_meta[cur]);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // The matrix instructions are assembly statements, so the compiler does not know that the
+    // accumulators come out of the matrix pipeline, and gives the copies it makes of them (from
+    // one accumulation register to another where the loop is left, into vector registers for
+    // the epilogue) none of the wait states such a read needs: placed right behind the last
+    // matrix instruction, a copy read the fourth register of an accumulator before that
+    // instruction had written it.  The wait states are spent explicitly wherever control can
+    // leave the straight run of steps: in statements that take every accumulator as an in-place
+    // operand, so that no copy of an accumulator's value can stand between the last matrix
+    // instruction and them; the first one holds the wait (32 clocks per three steps of ~2000).
+    auto settle = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        if (XT) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc_shared[0]), "+a"(acc_shared[1]));
+        else asm volatile("s_nop 15\n\ts_nop 15");
+#pragma unroll
+        for (int i = MI - 1; i >= 0; --i) {
+            static_assert(NTW == 4 || NTW == 5, "the accumulators of one row group in one statement");
+            if constexpr (NTW == 4)
+                asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]));
+            else
+                asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][NTW - 1]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // whole rotations of the three register sets in a loop, the last one or two steps after it
     uint32_t step = step_begin;
     for (; step + 3u <= step_end; step += 3u) {
         one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
         one_step(step + 1u, std::integral_constant<int, 1>(), std::integral_constant<int, 2>());
         one_step(step + 2u, std::integral_constant<int, 2>(), std::integral_constant<int, 0>());
+        settle();
     }
-    if (step < step_end) one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
-    if (step + 1u < step_end)
+    if (step < step_end) {
+        one_step(step, std::integral_constant<int, 0>(), std::integral_constant<int, 1>());
+        settle();
+    }
+    if (step + 1u < step_end) {
         one_step(step + 1u, std::integral_constant<int, 1>(), std::integral_constant<int, 2>());
-
-    // The matrix instructions are assembly statements, so the compiler does not know that the
-    // accumulators come out of the matrix pipeline, and gives the copies it makes of them into
-    // vector registers for the epilogue none of the wait states such a read needs: placed right
-    // behind the last matrix instruction, a copy read the fourth register of an accumulator
-    // before that instruction had written it.  The wait states are spent here, in statements
-    // that take every accumulator as an in-place operand, so that no copy of an accumulator's
-    // final value can stand before them; the first one holds the wait (the accumulators of the
-    // last slots are the ones still in the pipeline).
-    __builtin_amdgcn_sched_barrier(0);
-    if (XT) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc_shared[0]), "+a"(acc_shared[1]));
-    else asm volatile("s_nop 15\n\ts_nop 15");
-#pragma unroll
-    for (int i = MI - 1; i >= 0; --i) {
-        static_assert(NTW == 4 || NTW == 5, "the accumulators of one row group in one statement");
-        if constexpr (NTW == 4)
-            asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]));
-        else
-            asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][NTW - 1]));
+        settle();
     }
 
     // The spare fetches of the last steps land in LDS and in registers nobody reads: those
