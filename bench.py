@@ -508,6 +508,62 @@ def measure_w8a8(engine, ctx, steps, warmup, preheat_ms, with_cpu=True):
     return result
 
 
+Q8_AFFINE = {"N": 25600, "K": 5120}  # gate/up projection of the H3 text conditioner (minimax_h3_m3_e2e.m:2197-2205)
+
+
+def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
+    """Affine-Q8 g64 linear (minimax_h3_q8_gemm_bf16_meta's format) of the conditioner's gate shape:
+    GB/s of the weight image at M = 1, TFLOP/s at prefill M.  The weight is one Q4 weight of twice
+    the columns here (high nibbles | low nibbles) against the activations written twice, so a
+    linear is a small copy kernel and one Q4 linear.  Random codes and metadata: timing only,
+    parity is the GPU tests' business."""
+    N, K = Q8_AFFINE["N"], Q8_AFFINE["K"]
+    rng = np.random.default_rng(77)
+    quants = rng.integers(0, 256, size=N * K, dtype=np.uint8)
+    scales = (rng.random(N * (K // 64), dtype=np.float32) * 2e-4 + 2e-4)
+    biases = -scales * 128.0
+    to_bf16 = lambda v: (v.view(np.uint32) >> 16).astype(np.uint16)
+    weights = [ctx.q8_prepare(quants, to_bf16(scales), to_bf16(biases), N, K, engine.META_BF16_PLANES)
+               for _ in range(copies)]
+    image_bytes = N * K + N * (K // 64) * 4
+    out = {}
+    for M in rows_list:
+        x_ptr = ctx.to_device(engine.synth_normal_f16(5, 1.0, M * K).reshape(M, K))
+        y_ptr = ctx.alloc(M * N * 2)
+        state = {"i": 0}
+
+        def run_steps(n):
+            for _ in range(n):
+                ctx.q8_linear_device(weights[state["i"] % copies], x_ptr, engine.F16, M, y_ptr, engine.F16)
+                state["i"] += 1
+
+        steps = 60 if M == 1 else 20
+        timed = time_steps(ctx, run_steps, steps, 6, 20.0, preheat_batch=20)
+        kernel_s = timed["kernel_ms"] * 1e-3 / steps
+        entry = {"rows": M, "steps": steps, "launches_per_linear": timed["launches"] // steps,
+                 "kernel_us_per_linear": round(kernel_s * 1e6, 2),
+                 "wall_us_per_linear": round(timed["wall"] / steps * 1e6, 2)}
+        if M <= 16:
+            achieved = (image_bytes + M * K * 2 + M * N * 2) / kernel_s / 1e9
+            entry.update({"gb_per_s": round(achieved, 1),
+                          "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                                       "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                                       "kernel": "q4_stream_kernel over [high | low nibbles] x [x | x] (q8_double_x_kernel included)"}})
+        else:
+            achieved = 2.0 * M * N * K / kernel_s / 1e12
+            entry.update({"tflops": round(achieved, 1),
+                          "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": F16_MFMA_PEAK_TFLOPS,
+                                       "unit": "TFLOP/s", "frac": round(achieved / F16_MFMA_PEAK_TFLOPS, 4),
+                                       "kernel": "q4_gemm_pipe_kernel over [high | low nibbles] x [x | x]: the matrix "
+                                                 "units do 2x the algorithmic flops counted here"}})
+        out["q8_affine_g64_m%d" % M] = entry
+        ctx.free(x_ptr)
+        ctx.free(y_ptr)
+    for weight in weights:
+        ctx.q8_destroy(weight)
+    return out
+
+
 def bench_w8a8(engine, ctx, args):
     M, K, N, count = W8A8["M"], W8A8["K"], W8A8["N"], W8A8["projections"]
     r = measure_w8a8(engine, ctx, args.steps, args.warmup, args.preheat_ms, with_cpu=not args.no_cpu)
@@ -575,6 +631,7 @@ def secondary_figures(engine, ctx, work, args):
     if "cpu_baseline" in w:
         out["w8a8_m64_k1024_n4096"]["bit_exact_vs_oracle"] = w["bit_exact_vs_oracle"]
         out["w8a8_m64_k1024_n4096"]["cpu_baseline"] = w["cpu_baseline"]
+    out.update(measure_q8_affine(engine, ctx))
     return out
 
 
@@ -586,7 +643,7 @@ def main():
     parser.add_argument("--copies", type=int, default=8)
     parser.add_argument("--rows", type=int, default=None,
                         help="activation rows M (default 1; 512 for --workload prefill)")
-    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "lm_head", "prefill", "w8a8"])
+    parser.add_argument("--workload", default="layer_m1", choices=["layer_m1", "config1", "lm_head", "prefill", "w8a8", "q8"])
     parser.add_argument("--preheat-ms", type=float, default=100.0,
                         help="GPU time of untimed steps before anything is timed (0: none)")
     parser.add_argument("--unfused", action="store_true",
@@ -610,6 +667,10 @@ def main():
 
     if args.rows is None:
         args.rows = 512 if args.workload == "prefill" else 1
+    if args.workload == "q8":  # the affine-Q8 figures alone (for profiling); no line of the contract's shape
+        with engine.Context(0) as ctx:
+            print(json.dumps(measure_q8_affine(engine, ctx)), flush=True)
+        return 0
     if args.workload in ("prefill", "w8a8"):
         if args.steps == 400 and args.warmup == 40:
             args.steps, args.warmup = 100, 10

@@ -7,12 +7,14 @@
 //     scale * q + bias = (16 * scale) * hi + bias   +   scale * lo
 // and an affine-Q8 matrix is the sum of two affine-Q4 matrices over the same columns: one
 // with the high nibbles, scale 16*scale (a power-of-two multiple: exact) and the bias, one
-// with the low nibbles, the scale, and bias 0.  prepare splits the bytes once on the GPU
-// into two ordinary stream-tiled Q4 weights; a linear is the first one into an fp32
-// buffer and the second one with that buffer as its residual.  Every Q4 kernel, shape
-// heuristic and epilogue serves as is; the bytes read are the Q8 image's plus a second copy
-// of the metadata (+6 %).  The bias sits with the high part so that the GEMM path, which
-// rounds a weight to fp16, rounds the same magnitude the reference's half(scale*q+bias) does.
+// with the low nibbles, the scale, and bias 0.  Side by side they are ONE affine-Q4 matrix of
+// twice the columns, [high part | low part], applied to the activation row written twice,
+// [x | x].  prepare splits the bytes once on the GPU into that ordinary stream-tiled Q4
+// weight; a linear writes the activations twice into a staging buffer (one small kernel) and
+// runs one Q4 linear.  Every Q4 kernel, shape heuristic and epilogue serves as is; the bytes
+// read are the Q8 image's plus a second copy of the metadata (+6 %).  The bias sits with the
+// high part so that the GEMM path, which rounds a weight to fp16, rounds the same magnitude
+// the reference's half(scale*q+bias) does.
 #include "device_util.h"
 #include "internal.h"
 
@@ -22,14 +24,12 @@
 namespace mi355q {
 
 // One thread per eight codes: two output words (high and low nibbles in the Q4 source
-// layout, column k of eight at bits 4*(k%8)); threads of the first code word of a group
-// also write the group's two metadata pairs.
+// layout, column k of eight at bits 4*(k%8)) of the doubled matrix [N][2K]; threads of the
+// first code word of a group also write the group's two metadata pairs.
 __global__ void __launch_bounds__(256)
 q8_split_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ meta_a,
                 const uint16_t *__restrict__ meta_b, int meta_kind, uint32_t N, uint32_t K,
-                uint32_t *__restrict__ hi_codes, uint32_t *__restrict__ lo_codes,
-                uint16_t *__restrict__ hi_a, uint16_t *__restrict__ hi_b, uint16_t *__restrict__ lo_a,
-                uint16_t *__restrict__ lo_b)
+                uint32_t *__restrict__ codes, uint16_t *__restrict__ out_a, uint16_t *__restrict__ out_b)
 {
     const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t words = (uint64_t)N * (K / 8u);
@@ -42,36 +42,41 @@ q8_split_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__
         hi |= (byte >> 4) << (4u * c);
         lo |= (byte & 15u) << (4u * c);
     }
-    hi_codes[index] = hi;
-    lo_codes[index] = lo;
+    // row n of the doubled matrix: K/8 words of high nibbles, then K/8 words of low nibbles
+    const uint32_t words_per_row = K / 8u;
+    const uint64_t row = index / words_per_row, word = index % words_per_row;
+    codes[row * 2u * words_per_row + word] = hi;
+    codes[row * 2u * words_per_row + words_per_row + word] = lo;
     if (index % 8u != 0) return;
-    const uint64_t block = index / 8u;  // (row, group)
+    const uint64_t block = index / 8u;  // (row, group) of the source
+    const uint32_t groups_per_row = K / 64u;
+    const uint64_t hi_block = row * 2u * groups_per_row + word / 8u, lo_block = hi_block + groups_per_row;
     if (meta_kind == MI355Q_META_F16_INTERLEAVED) {
         const _Float16 scale = __builtin_bit_cast(_Float16, meta_a[2u * block]);
-        hi_a[2u * block] = __builtin_bit_cast(uint16_t, (_Float16)(scale * (_Float16)16.0f));
-        hi_a[2u * block + 1u] = meta_a[2u * block + 1u];
-        lo_a[2u * block] = meta_a[2u * block];
-        lo_a[2u * block + 1u] = 0;
+        out_a[2u * hi_block] = __builtin_bit_cast(uint16_t, (_Float16)(scale * (_Float16)16.0f));
+        out_a[2u * hi_block + 1u] = meta_a[2u * block + 1u];
+        out_a[2u * lo_block] = meta_a[2u * block];
+        out_a[2u * lo_block + 1u] = 0;
     } else {
         const float scale = __builtin_bit_cast(float, (uint32_t)meta_a[block] << 16);
-        hi_a[block] = (uint16_t)(__builtin_bit_cast(uint32_t, scale * 16.0f) >> 16);  // exact
-        hi_b[block] = meta_b[block];
-        lo_a[block] = meta_a[block];
-        lo_b[block] = 0;
+        out_a[hi_block] = (uint16_t)(__builtin_bit_cast(uint32_t, scale * 16.0f) >> 16);  // exact
+        out_b[hi_block] = meta_b[block];
+        out_a[lo_block] = meta_a[block];
+        out_b[lo_block] = 0;
     }
 }
 
 // Q8 rows: per output row an fp32 scale and K signed bytes, w = scale * v
 // (the MMO_Q8_ROW tensors of minimindo_thinker.c:84-86,112-122 and the Q8 payload of
-// minimindo_audio_encoder.c:90,216-217).  v + 128 = 16 * hi + lo gives two Q4 weights with
-// the integer metadata {16, -128} and {1, 0} (exact in bf16), whose sum is the exact integer
-// dot product; the row's fp32 scale multiplies the finished sum, as the reference does.
+// minimindo_audio_encoder.c:90,216-217).  v + 128 = 16 * hi + lo gives the two halves of the
+// doubled Q4 weight the integer metadata {16, -128} and {1, 0} (exact in bf16): its product
+// with [x | x] is the integer-weighted sum; the row's fp32 scale multiplies the finished sum,
+// as the reference does.
 // One thread per eight codes.
 __global__ void __launch_bounds__(256)
 q8rows_split_kernel(const uint8_t *__restrict__ records, uint32_t N, uint32_t K,
-                    uint32_t *__restrict__ hi_codes, uint32_t *__restrict__ lo_codes,
-                    uint16_t *__restrict__ hi_a, uint16_t *__restrict__ hi_b, uint16_t *__restrict__ lo_a,
-                    uint16_t *__restrict__ lo_b, float *__restrict__ row_scale)
+                    uint32_t *__restrict__ codes, uint16_t *__restrict__ out_a, uint16_t *__restrict__ out_b,
+                    float *__restrict__ row_scale)
 {
     const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t words_per_row = K / 8u;
@@ -85,18 +90,30 @@ q8rows_split_kernel(const uint8_t *__restrict__ records, uint32_t N, uint32_t K,
         hi |= (code >> 4) << (4u * c);
         lo |= (code & 15u) << (4u * c);
     }
-    hi_codes[index] = hi;
-    lo_codes[index] = lo;
+    codes[(uint64_t)row * 2u * words_per_row + word] = hi;
+    codes[(uint64_t)row * 2u * words_per_row + words_per_row + word] = lo;
     if (word % 8u == 0) {  // first word of a 64-column group
-        const uint64_t block = (uint64_t)row * (K / 64u) + word / 8u;
-        hi_a[block] = 0x4180;  // bf16 16
-        hi_b[block] = 0xc300;  // bf16 -128
-        lo_a[block] = 0x3f80;  // bf16 1
-        lo_b[block] = 0;
+        const uint64_t hi_block = (uint64_t)row * 2u * (K / 64u) + word / 8u, lo_block = hi_block + K / 64u;
+        out_a[hi_block] = 0x4180;  // bf16 16
+        out_b[hi_block] = 0xc300;  // bf16 -128
+        out_a[lo_block] = 0x3f80;  // bf16 1
+        out_b[lo_block] = 0;
     }
     if (word == 0)
         row_scale[row] = __builtin_bit_cast(float, (uint32_t)record[0] | (uint32_t)record[1] << 8 |
                                                        (uint32_t)record[2] << 16 | (uint32_t)record[3] << 24);
+}
+
+// out[m] = [x[m] | x[m]] in 16-byte pieces (a row of K elements is a whole number of them)
+__global__ void __launch_bounds__(256)
+q8_double_x_kernel(const uint4 *__restrict__ x, uint4 *__restrict__ out, uint32_t M, uint32_t pieces_per_row)
+{
+    const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= (size_t)M * pieces_per_row) return;
+    const size_t m = at / pieces_per_row, piece = at % pieces_per_row;
+    const uint4 value = x[at];
+    out[m * 2u * pieces_per_row + piece] = value;
+    out[m * 2u * pieces_per_row + pieces_per_row + piece] = value;
 }
 
 // y[m][n] = sum[m][n] * scale[n] (+ residual), one thread per element
@@ -118,7 +135,8 @@ using namespace mi355q;
 
 struct mi355q_q8_weight {
     mi355q_context *ctx;
-    mi355q_q4_weight *hi, *lo;
+    mi355q_q4_weight *doubled;  // [N][2K]: high-nibble part, then low-nibble part
+    uint32_t N, K;
     float *row_scale;  // Q8 rows: the fp32 scale of every output row (device); else null
     size_t image_bytes;
 };
@@ -126,8 +144,7 @@ struct mi355q_q8_weight {
 extern "C" void mi355q_q8_weight_destroy(mi355q_q8_weight *weight)
 {
     if (weight == nullptr) return;
-    mi355q_q4_weight_destroy(weight->hi);
-    mi355q_q4_weight_destroy(weight->lo);
+    mi355q_q4_weight_destroy(weight->doubled);
     if (weight->row_scale) (void)hipFree(weight->row_scale);
     delete weight;
 }
@@ -159,16 +176,15 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
     const size_t code_bytes = (size_t)N * K, nibble_bytes = code_bytes / 2u;
     const size_t plane_bytes = groups * 2u, meta_bytes = planes ? plane_bytes : 2u * plane_bytes;
     auto aligned = [](size_t bytes) { return (bytes + 255u) & ~(size_t)255u; };
-    // source image (when it comes from the host) | hi codes | lo codes | hi meta a, b | lo meta a, b
+    // source image (when it comes from the host) | codes of the doubled matrix | its metadata a, b
     const bool from_device = flags & MI355Q_SOURCE_DEVICE;
     size_t at = 0;
     const size_t at_quants = at;  at += from_device ? 0 : aligned(code_bytes);
     const size_t at_meta_a = at;  at += from_device ? 0 : aligned(meta_bytes);
     const size_t at_meta_b = at;  at += from_device || !planes ? 0 : aligned(meta_bytes);
-    const size_t at_hi = at;      at += aligned(nibble_bytes);
-    const size_t at_lo = at;      at += aligned(nibble_bytes);
-    size_t at_m[4];
-    for (int i = 0; i < 4; ++i) { at_m[i] = at; at += aligned(meta_bytes); }
+    const size_t at_codes = at;   at += aligned(2u * nibble_bytes);
+    size_t at_m[2];
+    for (int i = 0; i < 2; ++i) { at_m[i] = at; at += aligned(2u * meta_bytes); }
     char *scratch = nullptr;
     MI355Q_HIP(hipMalloc((void **)&scratch, at), "q8 conversion buffer");
     const void *d_quants = quants, *d_a = meta_a, *d_b = meta_b;
@@ -187,20 +203,16 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
         const uint64_t words = (uint64_t)N * (K / 8u);
         hipLaunchKernelGGL(q8_split_kernel, dim3((uint32_t)((words + 255u) / 256u)), dim3(256), 0, ctx->stream,
                            (const uint8_t *)d_quants, (const uint16_t *)d_a, (const uint16_t *)d_b, meta_kind, N, K,
-                           (uint32_t *)(scratch + at_hi), (uint32_t *)(scratch + at_lo),
-                           (uint16_t *)(scratch + at_m[0]), (uint16_t *)(scratch + at_m[1]),
-                           (uint16_t *)(scratch + at_m[2]), (uint16_t *)(scratch + at_m[3]));
+                           (uint32_t *)(scratch + at_codes), (uint16_t *)(scratch + at_m[0]),
+                           (uint16_t *)(scratch + at_m[1]));
         status = hipGetLastError();
     }
     int code = MI355Q_OK;
-    mi355q_q4_weight *hi = nullptr, *lo = nullptr;
+    mi355q_q4_weight *doubled = nullptr;
     if (status != hipSuccess) code = fail_hip(status, "q8 split", error, error_capacity);
     if (code == MI355Q_OK)  // stream order: the re-tiling kernels run after the split
-        code = mi355q_q4_weight_prepare(ctx, scratch + at_hi, scratch + at_m[0], planes ? scratch + at_m[1] : nullptr,
-                                        N, K, meta_kind, MI355Q_SOURCE_DEVICE, &hi, error, error_capacity);
-    if (code == MI355Q_OK)
-        code = mi355q_q4_weight_prepare(ctx, scratch + at_lo, scratch + at_m[2], planes ? scratch + at_m[3] : nullptr,
-                                        N, K, meta_kind, MI355Q_SOURCE_DEVICE, &lo, error, error_capacity);
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_codes, scratch + at_m[0], planes ? scratch + at_m[1] : nullptr,
+                                        N, 2u * K, meta_kind, MI355Q_SOURCE_DEVICE, &doubled, error, error_capacity);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(scratch);
     mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
@@ -209,13 +221,13 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
         code = MI355Q_ERROR_RUNTIME;
     }
     if (code != MI355Q_OK) {
-        mi355q_q4_weight_destroy(hi);
-        mi355q_q4_weight_destroy(lo);
+        mi355q_q4_weight_destroy(doubled);
         return code;
     }
     weight->ctx = ctx;
-    weight->hi = hi;
-    weight->lo = lo;
+    weight->doubled = doubled;
+    weight->N = N;
+    weight->K = K;
     weight->row_scale = nullptr;
     weight->image_bytes = code_bytes + groups * 4u;
     *out = weight;
@@ -242,10 +254,9 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
     auto aligned = [](size_t bytes) { return (bytes + 255u) & ~(size_t)255u; };
     const bool from_device = flags & MI355Q_SOURCE_DEVICE;
     size_t at = from_device ? 0 : aligned(record_bytes);
-    const size_t at_hi = at;  at += aligned(nibble_bytes);
-    const size_t at_lo = at;  at += aligned(nibble_bytes);
-    size_t at_m[4];
-    for (int i = 0; i < 4; ++i) { at_m[i] = at; at += aligned(plane_bytes); }
+    const size_t at_codes = at;  at += aligned(2u * nibble_bytes);
+    size_t at_m[2];
+    for (int i = 0; i < 2; ++i) { at_m[i] = at; at += aligned(2u * plane_bytes); }
     char *scratch = nullptr;
     float *row_scale = nullptr;
     MI355Q_HIP(hipMalloc((void **)&scratch, at), "q8 rows conversion buffer");
@@ -258,20 +269,17 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
     if (status == hipSuccess) {
         const uint64_t words = (uint64_t)N * (K / 8u);
         hipLaunchKernelGGL(q8rows_split_kernel, dim3((uint32_t)((words + 255u) / 256u)), dim3(256), 0, ctx->stream,
-                           source, N, K, (uint32_t *)(scratch + at_hi), (uint32_t *)(scratch + at_lo),
-                           (uint16_t *)(scratch + at_m[0]), (uint16_t *)(scratch + at_m[1]),
-                           (uint16_t *)(scratch + at_m[2]), (uint16_t *)(scratch + at_m[3]), row_scale);
+                           source, N, K, (uint32_t *)(scratch + at_codes), (uint16_t *)(scratch + at_m[0]),
+                           (uint16_t *)(scratch + at_m[1]), row_scale);
         status = hipGetLastError();
     }
     int code = MI355Q_OK;
-    mi355q_q4_weight *hi = nullptr, *lo = nullptr;
+    mi355q_q4_weight *doubled = nullptr;
     if (status != hipSuccess) code = fail_hip(status, "q8 rows split", error, error_capacity);
     if (code == MI355Q_OK)
-        code = mi355q_q4_weight_prepare(ctx, scratch + at_hi, scratch + at_m[0], scratch + at_m[1], N, K,
-                                        MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &hi, error, error_capacity);
-    if (code == MI355Q_OK)
-        code = mi355q_q4_weight_prepare(ctx, scratch + at_lo, scratch + at_m[2], scratch + at_m[3], N, K,
-                                        MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &lo, error, error_capacity);
+        code = mi355q_q4_weight_prepare(ctx, scratch + at_codes, scratch + at_m[0], scratch + at_m[1], N, 2u * K,
+                                        MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &doubled, error,
+                                        error_capacity);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(scratch);
     mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
@@ -280,14 +288,14 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
         code = MI355Q_ERROR_RUNTIME;
     }
     if (code != MI355Q_OK) {
-        mi355q_q4_weight_destroy(hi);
-        mi355q_q4_weight_destroy(lo);
+        mi355q_q4_weight_destroy(doubled);
         if (row_scale) (void)hipFree(row_scale);
         return code;
     }
     weight->ctx = ctx;
-    weight->hi = hi;
-    weight->lo = lo;
+    weight->doubled = doubled;
+    weight->N = N;
+    weight->K = K;
     weight->row_scale = row_scale;
     weight->image_bytes = record_bytes;
     *out = weight;
@@ -306,24 +314,48 @@ extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *wei
         set_error(error, error_capacity, "q8_linear: weight belongs to another context");
         return MI355Q_ERROR_INVALID;
     }
-    uint32_t N = 0;
-    mi355q_q4_weight_shape(weight->hi, &N, nullptr);
-    const size_t cells = (size_t)M * N;
-    const uint32_t keep = flags & (MI355Q_X_DEVICE | MI355Q_ASYNC);
-    if (weight->row_scale == nullptr) {
-        // the high part (+ the caller's residual) into fp32, then the low part on top of it
-        int status = ensure_stage(ctx, 5, cells * sizeof(float), error, error_capacity);
-        if (status != MI355Q_OK) return status;
-        void *partial = ctx->stage[5];
-        status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, residual, residual_dtype,
-                                  keep | MI355Q_Y_DEVICE |
-                                      (flags & (MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
-                                  error, error_capacity);
-        if (status != MI355Q_OK) return status;
-        return mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, y, y_dtype, partial, MI355Q_F32,
-                                keep | (flags & MI355Q_Y_DEVICE) | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+    if (!dtype_valid(x_dtype)) {
+        set_error(error, error_capacity, "q8_linear: x_dtype=%d", x_dtype);
+        return MI355Q_ERROR_INVALID;
     }
-    // Q8 rows: the integer sum of both parts in fp32, then scale (and residual) per element
+    const uint32_t N = weight->N, K = weight->K;
+    const size_t cells = (size_t)M * N;
+    const bool x_dev = flags & MI355Q_X_DEVICE;
+    if (x_dev && ((uintptr_t)x & 15u) != 0) {
+        set_error(error, error_capacity, "q8_linear: device x must be 16-byte aligned");
+        return MI355Q_ERROR_INVALID;
+    }
+    if ((flags & MI355Q_ASYNC) && !x_dev) {
+        set_error(error, error_capacity, "q8_linear: ASYNC needs device pointers throughout");
+        return MI355Q_ERROR_INVALID;
+    }
+    MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    // staging: [x as given, when it comes from the host | x twice per row | fp32 sums of the rows format]
+    const size_t x_bytes = (size_t)M * K * dtype_bytes(x_dtype);
+    const size_t at_given = 0, at_twice = x_dev ? 0 : (x_bytes + 255u) & ~(size_t)255u;
+    const size_t at_sum = at_twice + ((2u * x_bytes + 255u) & ~(size_t)255u);
+    int status = ensure_stage(ctx, 5, at_sum + (weight->row_scale ? cells * sizeof(float) : 0), error, error_capacity);
+    if (status != MI355Q_OK) return status;
+    char *stage = (char *)ctx->stage[5];
+    const void *x_on_device = x;
+    if (!x_dev) {
+        MI355Q_HIP(hipMemcpyAsync(stage + at_given, x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
+                   "activation upload");
+        x_on_device = stage + at_given;
+    }
+    {
+        const uint32_t pieces_per_row = (uint32_t)((size_t)K * dtype_bytes(x_dtype) / sizeof(uint4));
+        const size_t pieces = (size_t)M * pieces_per_row;
+        hipError_t launched = launch(ctx, q8_double_x_kernel, dim3((uint32_t)((pieces + 255u) / 256u)), dim3(256), 0,
+                                     (const uint4 *)x_on_device, (uint4 *)(stage + at_twice), M, pieces_per_row);
+        if (launched != hipSuccess) return fail_hip(launched, "q8 activation doubling launch", error, error_capacity);
+    }
+    const uint32_t keep = MI355Q_X_DEVICE | (flags & MI355Q_ASYNC);
+    if (weight->row_scale == nullptr)
+        return mi355q_q4_linear(ctx, weight->doubled, stage + at_twice, x_dtype, M, y, y_dtype, residual, residual_dtype,
+                                keep | (flags & (MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
+                                error, error_capacity);
+    // Q8 rows: the integer-weighted sum in fp32, then scale (and residual) per element
     if (!dtype_valid(y_dtype) || (residual != nullptr && !dtype_valid(residual_dtype))) {
         set_error(error, error_capacity, "q8_linear: y_dtype=%d residual_dtype=%d", y_dtype, residual_dtype);
         return MI355Q_ERROR_INVALID;
@@ -334,14 +366,9 @@ extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *wei
         set_error(error, error_capacity, "q8_linear: ASYNC needs device pointers throughout");
         return MI355Q_ERROR_INVALID;
     }
-    int status = ensure_stage(ctx, 5, 2u * cells * sizeof(float), error, error_capacity);
-    if (status != MI355Q_OK) return status;
-    float *partial = (float *)ctx->stage[5], *sum = partial + cells;
-    status = mi355q_q4_linear(ctx, weight->hi, x, x_dtype, M, partial, MI355Q_F32, nullptr, MI355Q_F32,
-                              keep | MI355Q_Y_DEVICE, error, error_capacity);
-    if (status != MI355Q_OK) return status;
-    status = mi355q_q4_linear(ctx, weight->lo, x, x_dtype, M, sum, MI355Q_F32, partial, MI355Q_F32,
-                              keep | MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE, error, error_capacity);
+    float *sum = (float *)(stage + at_sum);
+    status = mi355q_q4_linear(ctx, weight->doubled, stage + at_twice, x_dtype, M, sum, MI355Q_F32, nullptr, MI355Q_F32,
+                              MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC, error, error_capacity);
     if (status != MI355Q_OK) return status;
     const size_t y_bytes = cells * dtype_bytes(y_dtype);
     const size_t r_bytes = (is_bias ? N : cells) * dtype_bytes(residual_dtype);

@@ -354,6 +354,11 @@ class Context:
               _ptr(residual), residual_dtype, 0)
         return y
 
+    def q8_linear_device(self, weight, x_ptr: int, x_dtype: int, M: int, y_ptr: int, y_dtype: int = F32,
+                         asynchronous: bool = True):
+        _call(self.lib.mi355q_q8_linear, self.handle, weight, ctypes.c_void_p(x_ptr), x_dtype, M,
+              ctypes.c_void_p(y_ptr), y_dtype, None, F32, X_DEVICE | Y_DEVICE | (ASYNC if asynchronous else 0))
+
     def q38_image_open(self, image_bytes) -> Q38Image:
         """Opens the bytes of a .q38delta / .q38att / .q38global / .q38mtp file."""
         data = np.ascontiguousarray(np.frombuffer(image_bytes, dtype=np.uint8))

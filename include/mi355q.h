@@ -236,10 +236,11 @@ void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_
  * row n at byte (n * K/64 + g) * 64 + k), metadata as for Q4 (bf16 planes scales[N][K/64],
  * biases[N][K/64], or fp16 pairs): the projection format of minimax_h3_q8_gemm_bf16_meta
  * (minimax_h3_attention.metal:594-676).  prepare splits the codes into nibbles once:
- * scale*q + bias = (16*scale)*hi + bias + scale*lo, two ordinary Q4 weights, and
- * mi355q_q8_linear runs the two Q4 linears back to back (the second adds to the first in
- * fp32); arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the
- * GEMM path rounds each part to fp16 as the reference rounds half(scale*q + bias). */
+ * scale*q + bias = (16*scale)*hi + bias + scale*lo, i.e. one ordinary Q4 weight of twice
+ * the columns, [high part | low part]; mi355q_q8_linear writes every activation row twice
+ * ([x | x], one small kernel into a staging buffer) and runs one Q4 linear on it;
+ * arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the GEMM path
+ * rounds each part to fp16 as the reference rounds half(scale*q + bias). */
 typedef struct mi355q_q8_weight mi355q_q8_weight;
 int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
                              const void *meta_b, uint32_t N, uint32_t K, int meta_kind,
@@ -247,7 +248,7 @@ int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void
                              char *error, size_t error_capacity);
 /* Q8 rows: per output row an fp32 scale followed by K signed bytes, w = scale * v — the
  * MMO_Q8_ROW tensors of minimindo_thinker.c (:84-86,112-122) and the Q8 payload of
- * minimindo_audio_encoder.c (:90,216-217), records [N][4 + K].  Prepared as two Q4 weights
+ * minimindo_audio_encoder.c (:90,216-217), records [N][4 + K].  Prepared the same way
  * with integer metadata (v + 128 = 16*hi + lo), so mi355q_q8_linear on such a weight
  * computes the exact integer-weighted sum in fp32 and multiplies it by the row's scale at
  * the end, as q8_f32_dot's callers do (minimindo_thinker.c:124-213, q8_matvec /
