@@ -290,8 +290,10 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
                 typedef const __attribute__((address_space(1))) char *global_bytes;
                 const u32x4 q = __builtin_nontemporal_load(
                     (const __attribute__((address_space(1))) u32x4 *)((global_bytes)codes_at + codes_lane[tb]));
-                const u32x2 m = __builtin_nontemporal_load(
-                    (const __attribute__((address_space(1))) u32x2 *)((global_bytes)meta_at + meta_lane[tb]));
+                // the metadata with an ordinary load: its four lane groups read the same 128 bytes, and
+                // without the streaming hint the vector cache answers three of them (layer at
+                // M = 1: 1.3 % faster, the same at M = 8)
+                const u32x2 m = *(const __attribute__((address_space(1))) u32x2 *)((global_bytes)meta_at + meta_lane[tb]);
                 slot.q[tb] = make_uint4(q.x, q.y, q.z, q.w);
                 slot.m[tb] = make_uint2(m.x, m.y);
             }
