@@ -1036,7 +1036,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     // faster than a full one: the chip is power limited, and up to about half of it the clock
     // stays near its maximum, from there it falls to the sustained clock of a full chip
     // (fitted, like the other figures here, to interleaved timings of every variant and split
-    // at M = 256 .. 4096 on the 27B shapes: 4 % rms, the fastest choice found in 13 of 14 cases).
+    // at M = 128 .. 4096 on the 27B shapes: 3 % rms over 78 timings of the pipelined variants).
     auto partial_round = [](double r) {
         const double over = (1.0 - r) / 0.438;
         return r <= 0.562 ? 0.771 - 0.081 * r / 0.562 : 1.0 - 0.31 * over * over;
@@ -1065,12 +1065,11 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             const double peak_us = (double)steps * tiles_per_wave * (c.bm / 16.0) * 64.0 / 2400.0;
             double cost;
             if (v >= 6) {
-                // 7.6 us per launch; a round = 7.2 us (fill, and the burst of stores at its end)
+                // 6.0 us per launch; a round = 5.5 us (fill, and the burst of stores at its end)
                 // plus its steps
                 const uint64_t rest = groups % cus;
-                const double round = 7.2 + (double)steps * c.step_us;
-                cost = 7.6 + round * ((double)(groups / cus) + (rest ? partial_round((double)rest / cus) : 0.0));
-                if (splits > 1 && c.ntw == 5) cost += 0.07 * steps * c.step_us;  // 20 tiles of fp32 to write
+                const double round = 5.5 + (double)steps * c.step_us;
+                cost = 6.0 + round * ((double)(groups / cus) + (rest ? partial_round((double)rest / cus) : 0.0));
             }
             else if (groups <= cus)
                 cost = peak_us / c.alone;
@@ -1083,7 +1082,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             else
                 cost = ((double)groups / slots + (groups % slots ? 0.31 : 0.0)) * c.resident * peak_us / c.shared;
             if (splits > 1)  // fp32 partials at 4.6 TB/s and the kernel that adds them
-                cost += (double)splits * a.M * (double)w.N * 4.0 / 4.63e6 + 6.3;
+                cost += (double)splits * a.M * (double)w.N * 4.0 / 4.63e6 + (v >= 6 ? 2.0 : 6.3);
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;
