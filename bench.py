@@ -514,8 +514,8 @@ Q8_AFFINE = {"N": 25600, "K": 5120}  # gate/up projection of the H3 text conditi
 def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
     """Affine-Q8 g64 linear (minimax_h3_q8_gemm_bf16_meta's format) of the conditioner's gate shape:
     GB/s of the weight image at M = 1, TFLOP/s at prefill M.  The weight is one Q4 weight of twice
-    the columns here (high nibbles | low nibbles) against the activations written twice, so a
-    linear is a small copy kernel and one Q4 linear.  Random codes and metadata: timing only,
+    the columns here (high nibbles | low nibbles) whose second half meets the activation row again
+    from its start, so a linear is one Q4 linear.  Random codes and metadata: timing only,
     parity is the GPU tests' business."""
     N, K = Q8_AFFINE["N"], Q8_AFFINE["K"]
     rng = np.random.default_rng(77)
@@ -548,7 +548,7 @@ def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
             entry.update({"gb_per_s": round(achieved, 1),
                           "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                                       "kernel": "q4_stream_kernel over [high | low nibbles] x [x | x] (q8_double_x_kernel included)"}})
+                                       "kernel": "q4_stream_kernel over [high | low nibbles] x [x | x]"}})
         else:
             achieved = 2.0 * M * N * K / kernel_s / 1e12
             entry.update({"tflops": round(achieved, 1),

@@ -652,6 +652,20 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
                            const void *x, int x_dtype, uint32_t M, int y_dtype, int residual_dtype,
                            uint32_t flags, char *error, size_t error_capacity)
 {
+    return q4_linear_multi_repeated(ctx, targets, count, x, x_dtype, M, y_dtype, residual_dtype, flags, 0, error,
+                                    error_capacity);
+}
+
+}  // extern "C"
+
+namespace mi355q {
+
+// mi355q_q4_linear_multi with activation rows of x_columns columns that the weight's second
+// half of columns meets again (x_columns = K / 2, one target); 0: rows of K columns.
+int q4_linear_multi_repeated(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count,
+                             const void *x, int x_dtype, uint32_t M, int y_dtype, int residual_dtype,
+                             uint32_t flags, uint32_t x_columns, char *error, size_t error_capacity)
+{
     if (ctx == nullptr || targets == nullptr || x == nullptr || count == 0 || count > kMaxTargets) {
         set_error(error, error_capacity, "q4_linear: null argument or target count outside 1..%u",
                   kMaxTargets);
@@ -706,7 +720,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
         return MI355Q_ERROR_INVALID;
     }
     MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
-    const uint32_t K = targets[0].weight->dev.K;
+    const uint32_t K = x_columns ? x_columns : targets[0].weight->dev.K;
     const size_t x_bytes = (size_t)M * K * dtype_bytes(x_dtype);
     // host outputs / residuals are staged back to back, each 256-byte aligned
     size_t y_offset[kMaxTargets], r_offset[kMaxTargets], y_total = 0, r_total = 0;
@@ -730,6 +744,7 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
     args.residual_is_bias = is_bias;
     args.fuse_silu = fuse;
     args.count = count;
+    args.x_columns = x_columns;
     int status;
     if (!x_dev) {
         if ((status = ensure_stage(ctx, 0, x_bytes, error, error_capacity)) != MI355Q_OK) return status;
@@ -776,6 +791,10 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
         MI355Q_HIP(hipStreamSynchronize(ctx->stream), "q4_linear sync");
     return MI355Q_OK;
 }
+
+}  // namespace mi355q
+
+extern "C" {
 
 int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight, const void *x,
                      int x_dtype, uint32_t M, void *y, int y_dtype, const void *residual,

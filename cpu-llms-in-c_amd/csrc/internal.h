@@ -177,11 +177,19 @@ struct Q4LinearArgs {
     // live in the library's fixed device array (q4_stream_scratch_init), sizes beyond it are
     // refused, and so is per-kernel profiling (which creates events).
     bool no_alloc;
+    // Columns of an activation row when they are fewer than the weight's: K / 2 (a multiple of
+    // 128, one target).  The weight's second half of columns then meets the same row again from
+    // its start - how the doubled [high | low nibble] weight of an 8-bit matrix is applied.  0: K.
+    uint32_t x_columns;
 };
 // Looks up the device address of the fixed scratch array on the context's device (once per
 // device) and keeps it in the context; called by mi355q_context_create with that device current.
 hipError_t q4_stream_scratch_init(mi355q_context *ctx);
 int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity);
+// mi355q_q4_linear_multi with Q4LinearArgs::x_columns
+int q4_linear_multi_repeated(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count, const void *x,
+                             int x_dtype, uint32_t M, int y_dtype, int residual_dtype, uint32_t flags,
+                             uint32_t x_columns, char *error, size_t error_capacity);
 // q4_gemm.hip (one target at a time: `target` selects it)
 int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, char *error,
                    size_t error_capacity);

@@ -38,6 +38,9 @@ struct GemmParams {
     const uint4 *codes;
     const uint2 *meta;
     const _Float16 *x;  // [M][K] fp16
+    // K: columns of an activation row - the weight's, unless the weight's steps from wrap_steps on
+    // meet the row again from its start (then x has wrap_steps * 128 columns); 0xffffffff: never
+    uint32_t wrap_steps;
     void *y;
     const void *residual;
     float *partials;    // [splits][M][N] when splits > 1
@@ -211,7 +214,7 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
             // the octet is already in a_source; only the K tail needs care: when K is an odd
             // multiple of 64 the upper half of the last step does not exist, and the lane
             // reads the lower half again (64 columns back, still inside its row)
-            const uint32_t k = step * kStepColumns;
+            const uint32_t k = (step >= p.wrap_steps ? step - p.wrap_steps : step) * kStepColumns;
             const uint32_t octet = r ^ (((BM / 4) * wave + 4u * j + kq) & 15u);
             const _Float16 *source = a_source[j] + k;
             if (k + 8u * octet >= p.K) source -= 64;
@@ -534,7 +537,8 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     }
     const uint32_t last_step = step_end - 1u;
     // the fetch pointers: they stop at the last step (later fetches repeat it: no branches)
-    const char *x_next = (const char *)(p.x + (size_t)step_begin * kStepColumns) - 4096;
+    const char *x_next =
+        (const char *)(p.x + (size_t)(step_begin >= p.wrap_steps ? step_begin - p.wrap_steps : step_begin) * kStepColumns) - 4096;
     const char *codes_next = (const char *)(p.codes + (size_t)step_begin * p.NT * 64u);
     const char *meta_next = (const char *)(p.meta + (size_t)step_begin * p.NT * 16u);
     uint32_t fetch_step = step_begin;
@@ -568,6 +572,8 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         const bool more = fetch_step < last_step;
         fetch_step += 1u;
         x_next += more ? kStepColumns * sizeof(_Float16) : 0u;
+        if (more && fetch_step == p.wrap_steps)  // the activation row starts over
+            x_next -= (size_t)p.wrap_steps * (kStepColumns * sizeof(_Float16));
         codes_next += more ? codes_stride : 0u;
         meta_next += more ? meta_stride : 0u;
     };
@@ -990,8 +996,13 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     p.codes = w.codes;
     p.meta = w.meta16;  // fp16 {scale, bias}: the weight is evaluated in fp16 here
     p.x = (const _Float16 *)a.x;
+    if (a.x_columns != 0 && (a.x_columns * 2u != w.K || a.x_columns % kStepColumns != 0)) {
+        set_error(error, error_capacity, "q4 gemm: a repeated activation row is half the weight's columns, whole 128-column steps");
+        return MI355Q_ERROR_INVALID;
+    }
+    const uint32_t x_columns = a.x_columns ? a.x_columns : w.K;
     if (a.x_dtype != MI355Q_F16) {
-        const size_t count = (size_t)a.M * w.K;
+        const size_t count = (size_t)a.M * x_columns;
         int status = ensure_stage(ctx, 3, count * sizeof(_Float16), error, error_capacity);
         if (status != MI355Q_OK) return status;
         hipError_t converted =
@@ -1005,7 +1016,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     p.residual = a.targets[target].residual;
     p.M = a.M;
     p.N = w.N;
-    p.K = w.K;
+    p.K = x_columns;
+    p.wrap_steps = a.x_columns ? a.x_columns / kStepColumns : 0xffffffffu;
     p.NT = w.NT;
     p.T = w.T;
     p.y_dtype = a.y_dtype;
@@ -1046,7 +1058,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     uint32_t best_splits = 1;
     double best_cost = 1e30;
     // the pipelined kernel addresses x with 32-bit byte offsets and whole 128-column steps
-    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * w.K * sizeof(_Float16) + 16384u < (1ull << 32);
+    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
         if (v >= 6 && !pipe_ok) continue;
         const Variant &c = variants[v];

@@ -106,7 +106,10 @@ struct StreamParams {
     // that brings the row's largest magnitude to [2^13, 2^14); row_scale[m] is the inverse power,
     // by which the finished dot products of row m are multiplied.  Null: fp16 activations as given.
     const float *row_scale;
-    uint32_t M, K, T;
+    uint32_t M, K, T;      // K: columns of an activation row (the weight's, except as below)
+    // the weight's steps from wrap_steps on meet the activation row again from its start
+    // (x has wrap_steps * 128 columns); 0xffffffff: never
+    uint32_t wrap_steps;
     uint32_t rows;         // M, or 2*M when fp32 activations are carried as (value, remainder) pairs
     // The T steps are cut in `slices` runs of slice_steps (workgroups with blockIdx.y == s
     // take run s).  With more than one slice the workgroups write fp32
@@ -141,7 +144,10 @@ struct StepData {
     uint2 m[TB];
 };
 
-template <int MP, int TB, int D, int W, bool BF>
+// WRAP: the weight's steps from p.wrap_steps on meet the activation row again from its start (a
+// separate instantiation: the kernel for ordinary weights stays instruction for instruction what
+// it was; its sixteen-wave form fits two workgroups on a compute unit only below 65 registers)
+template <int MP, int TB, int D, int W, bool BF, bool WRAP = false>
 __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
 {
     extern __shared__ uint4 lds[];
@@ -157,6 +163,7 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     const uint32_t columns = p.columns, targets = p.targets, first1 = p.first_block[1],
                    first2 = p.first_block[2], first3 = p.first_block[3];
     const uint32_t T = p.T, K = p.K, slice_steps = p.slice_steps, rows = p.rows;
+    const uint32_t wrap_steps = WRAP ? p.wrap_steps : 0xffffffffu;
     const int fuse_silu = p.fuse_silu;
     const uint32_t *const ids = p.ids;
     const _Float16 *const x = p.x;
@@ -262,7 +269,8 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
         // "everything up to the n-th newest fetch has landed".
         auto fetch = [&](uint32_t step, auto slot_c, StepData<TB> &slot) {
             constexpr uint32_t slot_bytes = decltype(slot_c)::value * SLAB * (uint32_t)sizeof(uint4);
-            uint64_t x_at = (uint64_t)((const char *)x + (size_t)step * (kStepColumns * sizeof(_Float16)));
+            const uint32_t x_step = WRAP && step >= wrap_steps ? step - wrap_steps : step;
+            uint64_t x_at = (uint64_t)((const char *)x + (size_t)x_step * (kStepColumns * sizeof(_Float16)));
             asm volatile("" : "+s"(x_at));
             const bool tail_step = odd_tail && step + 1u == T;
 #pragma unroll
@@ -666,6 +674,11 @@ static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
     // when the row of workgroups in front of each slice is a whole number of rounds over the XCDs
     const uint32_t xcds = 8;
     const dim3 grid(q.arrivals ? (blocks + xcds - 1) / xcds * xcds : blocks, q.slices);
+    if (q.wrap_steps != 0xffffffffu) {
+        if (q.meta_bf16)
+            return launch(ctx, q4_stream_kernel<MP, TB, D, W, true, true>, grid, dim3(64u * W), lds, q);
+        return launch(ctx, q4_stream_kernel<MP, TB, D, W, false, true>, grid, dim3(64u * W), lds, q);
+    }
     if (q.meta_bf16)
         return launch(ctx, q4_stream_kernel<MP, TB, D, W, true>, grid, dim3(64u * W), lds, q);
     return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, grid, dim3(64u * W), lds, q);
@@ -768,6 +781,12 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     }
     int mp = 1;
     while ((uint32_t)mp < rows) mp *= 2;
+    if (a.x_columns != 0 && (a.count != 1 || a.x_columns * 2u != first.K || a.x_columns % kStepColumns != 0)) {
+        set_error(error, error_capacity, "q4 stream kernel: a repeated activation row is half the weight's columns, "
+                                         "whole 128-column steps, one target");
+        return MI355Q_ERROR_INVALID;
+    }
+    const uint32_t x_columns = a.x_columns ? a.x_columns : first.K;
 
     StreamParams p;
     memset(&p, 0, sizeof p);
@@ -779,7 +798,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     }
     if (a.x_dtype != MI355Q_F16) {
         // [ the rows' inverse scales (16 floats, 256 bytes) | rows * K fp16 ]
-        const size_t bytes = kRowScaleBytes + (size_t)rows * first.K * sizeof(_Float16);
+        const size_t bytes = kRowScaleBytes + (size_t)rows * x_columns * sizeof(_Float16);
         unsigned char *area;
         if (a.no_alloc) {
             if (bytes > kScratchXBytes) {
@@ -796,7 +815,7 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
         float *const row_scale = (float *)area;
         _Float16 *const converted_x = (_Float16 *)(area + kRowScaleBytes);
         hipError_t converted = launch(ctx, q4_convert_x_kernel, dim3(a.M), dim3(kConvertThreads), 0, a.x,
-                                      a.x_dtype, converted_x, row_scale, a.M, first.K);
+                                      a.x_dtype, converted_x, row_scale, a.M, x_columns);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = converted_x;
@@ -836,8 +855,9 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     p.matrix_rows = first.N;
     p.targets = a.count;
     p.M = a.M;
-    p.K = first.K;
+    p.K = x_columns;
     p.T = first.T;
+    p.wrap_steps = a.x_columns ? a.x_columns / kStepColumns : 0xffffffffu;
     p.rows = rows;
     p.slice_steps = shape.slice_steps;
     p.slices = shape.slices;

@@ -8,10 +8,11 @@
 // and an affine-Q8 matrix is the sum of two affine-Q4 matrices over the same columns: one
 // with the high nibbles, scale 16*scale (a power-of-two multiple: exact) and the bias, one
 // with the low nibbles, the scale, and bias 0.  Side by side they are ONE affine-Q4 matrix of
-// twice the columns, [high part | low part], applied to the activation row written twice,
+// twice the columns, [high part | low part], applied to the activation row taken twice,
 // [x | x].  prepare splits the bytes once on the GPU into that ordinary stream-tiled Q4
-// weight; a linear writes the activations twice into a staging buffer (one small kernel) and
-// runs one Q4 linear.  Every Q4 kernel, shape heuristic and epilogue serves as is; the bytes
+// weight; a linear is one Q4 linear whose kernels start the activation row over at the
+// weight's second half (K a multiple of 128; otherwise one small kernel first writes the rows
+// twice into a staging buffer).  Every Q4 kernel, shape heuristic and epilogue serves as is; the bytes
 // read are the Q8 image's plus a second copy of the metadata (+6 %).  The bias sits with the
 // high part so that the GEMM path, which rounds a weight to fp16, rounds the same magnitude
 // the reference's half(scale*q+bias) does.
@@ -330,31 +331,44 @@ extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *wei
         return MI355Q_ERROR_INVALID;
     }
     MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+    // When K is a whole number of 128-column steps the Q4 kernels read the row twice themselves
+    // (the weight's second half of columns meets x again from its start); otherwise the rows are
+    // written twice into a staging buffer first.
     // staging: [x as given, when it comes from the host | x twice per row | fp32 sums of the rows format]
+    const bool repeat_in_kernel = K % 128u == 0;
     const size_t x_bytes = (size_t)M * K * dtype_bytes(x_dtype);
-    const size_t at_given = 0, at_twice = x_dev ? 0 : (x_bytes + 255u) & ~(size_t)255u;
-    const size_t at_sum = at_twice + ((2u * x_bytes + 255u) & ~(size_t)255u);
-    int status = ensure_stage(ctx, 5, at_sum + (weight->row_scale ? cells * sizeof(float) : 0), error, error_capacity);
+    const size_t at_given = 0, at_twice = x_dev || repeat_in_kernel ? 0 : (x_bytes + 255u) & ~(size_t)255u;
+    const size_t at_sum = repeat_in_kernel ? 0 : at_twice + ((2u * x_bytes + 255u) & ~(size_t)255u);
+    int status = MI355Q_OK;
+    if (!repeat_in_kernel || weight->row_scale)
+        status = ensure_stage(ctx, 5, at_sum + (weight->row_scale ? cells * sizeof(float) : 0), error, error_capacity);
     if (status != MI355Q_OK) return status;
     char *stage = (char *)ctx->stage[5];
-    const void *x_on_device = x;
-    if (!x_dev) {
-        MI355Q_HIP(hipMemcpyAsync(stage + at_given, x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
-                   "activation upload");
-        x_on_device = stage + at_given;
-    }
-    {
+    const void *x_for_linear = x;
+    uint32_t x_flags = flags & MI355Q_X_DEVICE;
+    if (!repeat_in_kernel) {
+        const void *x_on_device = x;
+        if (!x_dev) {
+            MI355Q_HIP(hipMemcpyAsync(stage + at_given, x, x_bytes, hipMemcpyHostToDevice, ctx->stream),
+                       "activation upload");
+            x_on_device = stage + at_given;
+        }
         const uint32_t pieces_per_row = (uint32_t)((size_t)K * dtype_bytes(x_dtype) / sizeof(uint4));
         const size_t pieces = (size_t)M * pieces_per_row;
         hipError_t launched = launch(ctx, q8_double_x_kernel, dim3((uint32_t)((pieces + 255u) / 256u)), dim3(256), 0,
                                      (const uint4 *)x_on_device, (uint4 *)(stage + at_twice), M, pieces_per_row);
         if (launched != hipSuccess) return fail_hip(launched, "q8 activation doubling launch", error, error_capacity);
+        x_for_linear = stage + at_twice;
+        x_flags = MI355Q_X_DEVICE;
     }
-    const uint32_t keep = MI355Q_X_DEVICE | (flags & MI355Q_ASYNC);
-    if (weight->row_scale == nullptr)
-        return mi355q_q4_linear(ctx, weight->doubled, stage + at_twice, x_dtype, M, y, y_dtype, residual, residual_dtype,
-                                keep | (flags & (MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE | MI355Q_RESIDUAL_IS_BIAS)),
-                                error, error_capacity);
+    const uint32_t x_columns = repeat_in_kernel ? K : 0u;
+    if (weight->row_scale == nullptr) {
+        const mi355q_q4_target target = {weight->doubled, y, residual};
+        return q4_linear_multi_repeated(ctx, &target, 1, x_for_linear, x_dtype, M, y_dtype, residual_dtype,
+                                        x_flags | (flags & (MI355Q_ASYNC | MI355Q_Y_DEVICE | MI355Q_RESIDUAL_DEVICE |
+                                                            MI355Q_RESIDUAL_IS_BIAS)),
+                                        x_columns, error, error_capacity);
+    }
     // Q8 rows: the integer-weighted sum in fp32, then scale (and residual) per element
     if (!dtype_valid(y_dtype) || (residual != nullptr && !dtype_valid(residual_dtype))) {
         set_error(error, error_capacity, "q8_linear: y_dtype=%d residual_dtype=%d", y_dtype, residual_dtype);
@@ -367,8 +381,13 @@ extern "C" int mi355q_q8_linear(mi355q_context *ctx, const mi355q_q8_weight *wei
         return MI355Q_ERROR_INVALID;
     }
     float *sum = (float *)(stage + at_sum);
-    status = mi355q_q4_linear(ctx, weight->doubled, stage + at_twice, x_dtype, M, sum, MI355Q_F32, nullptr, MI355Q_F32,
-                              MI355Q_X_DEVICE | MI355Q_Y_DEVICE | MI355Q_ASYNC, error, error_capacity);
+    {
+        // (a host x is uploaded by the linear itself, which then may not be told to return early)
+        const mi355q_q4_target target = {weight->doubled, sum, nullptr};
+        status = q4_linear_multi_repeated(ctx, &target, 1, x_for_linear, x_dtype, M, MI355Q_F32, MI355Q_F32,
+                                          x_flags | MI355Q_Y_DEVICE | (x_flags ? MI355Q_ASYNC : 0u), x_columns, error,
+                                          error_capacity);
+    }
     if (status != MI355Q_OK) return status;
     const size_t y_bytes = cells * dtype_bytes(y_dtype);
     const size_t r_bytes = (is_bias ? N : cells) * dtype_bytes(residual_dtype);

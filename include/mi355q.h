@@ -237,9 +237,10 @@ void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_
  * biases[N][K/64], or fp16 pairs): the projection format of minimax_h3_q8_gemm_bf16_meta
  * (minimax_h3_attention.metal:594-676).  prepare splits the codes into nibbles once:
  * scale*q + bias = (16*scale)*hi + bias + scale*lo, i.e. one ordinary Q4 weight of twice
- * the columns, [high part | low part]; mi355q_q8_linear writes every activation row twice
- * ([x | x], one small kernel into a staging buffer) and runs one Q4 linear on it;
- * arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the GEMM path
+ * the columns, [high part | low part], which mi355q_q8_linear applies to [x | x] in one Q4
+ * linear: the kernels start the activation row over at the weight's second half (K a
+ * multiple of 128; otherwise a small kernel first writes the rows twice into a staging
+ * buffer); arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the GEMM path
  * rounds each part to fp16 as the reference rounds half(scale*q + bias). */
 typedef struct mi355q_q8_weight mi355q_q8_weight;
 int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
