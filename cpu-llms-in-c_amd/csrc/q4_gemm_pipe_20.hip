@@ -1,0 +1,9 @@
+// The pipelined affine-Q4 GEMM kernel, 20 tiles per workgroup: one instantiation per file so that they
+// compile side by side.
+#include "q4_gemm_device.h"
+
+namespace mi355q {
+
+template __global__ void q4_gemm_pipe_kernel<128, 5, false, false>(const GemmParams);
+
+}  // namespace mi355q
