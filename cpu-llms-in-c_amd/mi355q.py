@@ -329,7 +329,7 @@ class Context:
               flags, ctypes.byref(out))
         return Q4Weight(self, out, N, K)
 
-    # ---- affine Q8 (two Q4 weights) ----
+    # ---- affine Q8 (one Q4 weight of twice the columns) ----
     def q8_prepare(self, quants, meta_a, meta_b, N: int, K: int, meta_kind: int):
         out = ctypes.c_void_p()
         _call(self.lib.mi355q_q8_weight_prepare, self.handle, _ptr(quants), _ptr(meta_a), _ptr(meta_b), N, K,

@@ -1,4 +1,4 @@
-"""GPU parity of the affine-Q8 g64 linear (two Q4 weights, mi355q_q8_linear) against the oracle.
+"""GPU parity of the affine-Q8 g64 linear (one Q4 weight of twice the columns, mi355q_q8_linear) against the oracle.
 
 Format and reference arithmetic: minimax_h3_q8_gemm_bf16_meta (minimax_h3_attention.metal:594-676),
 u8 quants[N][K], bf16 scales/biases [N][K/64], weight = scale * q + bias.
@@ -39,7 +39,11 @@ def make_q8(engine, seed, N, K, meta_kind):
 
 @pytest.mark.parametrize("N,K,M,meta", [(100, 192, 1, "META_BF16_PLANES"), (256, 1024, 1, "META_F16_INTERLEAVED"),
                                         (1024, 3072, 4, "META_BF16_PLANES"), (320, 8704, 8, "META_BF16_PLANES"),
-                                        (528, 1536, 64, "META_BF16_PLANES"), (1088, 640, 200, "META_F16_INTERLEAVED")])
+                                        (528, 1536, 64, "META_BF16_PLANES"), (1088, 640, 200, "META_F16_INTERLEAVED"),
+                                        # K not a whole number of 128-column steps: the rows are written twice first
+                                        (272, 320, 40, "META_BF16_PLANES"),
+                                        # long rows, K splits: the activation row starts over inside a split
+                                        (560, 2176, 150, "META_BF16_PLANES")])
 def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
     meta_kind = getattr(engine, meta)
     quants, meta_a, meta_b = make_q8(engine, 3, N, K, meta_kind)
