@@ -129,3 +129,24 @@ def test_q8rows_f32_shapes(engine, oracle, gpu, N, K, M):
         rms = np.sqrt(np.mean(ref * ref, axis=1, keepdims=True))
         assert float(np.max(np.abs(y - ref) / rms)) <= 2e-3
         assert float(np.max(np.abs(biased - (ref + bias)) / rms)) <= 2e-3
+
+
+@pytest.mark.parametrize("forced", ["0,1", "2,2", "3,1", "6,1", "6,3", "7,2", "8,2"])
+def test_q8_affine_under_every_gemm_kernel(engine, oracle, gpu, forced, force):
+    """The activation row starts over at the weight's second half of columns in each of the three
+    matrix kernels' addressing; every GEMM variant (first kernel, pipelined 16 / 17 / 20 tiles,
+    with and without K splits) on a Q8 weight whose doubled row is ten steps long."""
+    force("q4_gemm", forced)
+    N, K, M = 560, 640, 150
+    meta_kind = engine.META_BF16_PLANES
+    quants, meta_a, meta_b = make_q8(engine, 11, N, K, meta_kind)
+    x = np.stack([engine.synth_normal_f32(170 + m, 1.0, K) for m in range(M)]).astype(np.float16)
+    weight = gpu.q8_prepare(quants, meta_a, meta_b, N, K, meta_kind)
+    try:
+        print(f"q8 affine forced={forced}", flush=True)
+        y = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
+    finally:
+        gpu.q8_destroy(weight)
+    exact = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, engine.F16, M)
+    rms = np.sqrt(np.mean(exact * exact, axis=1, keepdims=True))
+    assert float(np.max(np.abs(y - exact) / rms)) <= 2e-3
