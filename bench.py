@@ -623,6 +623,11 @@ def secondary_figures(engine, ctx, work, args):
                            "algorithmic_flops_per_step": p["step_flops"], "roofline": p["roofline"]}
     if "cpu_baseline" in p:
         out["prefill_m512"]["cpu_baseline"] = p["cpu_baseline"]
+    # the same three linears at M = 2048 (the shape divides evenly over the compute units from there on)
+    p = measure_prefill(engine, ctx, 2048, 10, 3, 20.0, weights=mlp, host=host, with_cpu=False)
+    out["prefill_m2048"] = {"tflops": p["tflops"], "percent_of_f16_peak": p["percent_of_f16_peak"],
+                            "steps": 10, "warmup": 3, "linears_per_step": 3,
+                            "algorithmic_flops_per_step": p["step_flops"], "roofline": p["roofline"]}
     w = measure_w8a8(engine, ctx, 200, 20, 20.0, with_cpu=not args.no_cpu)
     out["w8a8_m64_k1024_n4096"] = {"tops": w["tops"], "steps": 200, "warmup": 20, "projections_per_step": 3,
                                    "projection_launch_us_p50": w["projection_launch_us_p50"],
