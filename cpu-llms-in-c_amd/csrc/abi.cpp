@@ -43,6 +43,18 @@ int ensure_stage(mi355q_context *ctx, int slot, size_t bytes, char *error,
     return MI355Q_OK;
 }
 
+int chain_after_wait(mi355q_context *ctx, char *error, size_t error_capacity)
+{
+    if (!ctx->chain_pending) return MI355Q_OK;
+    ctx->chain_pending = false;
+    if (ctx->chain_gave_up == nullptr || *(volatile uint32_t *)ctx->chain_gave_up == 0u) return MI355Q_OK;
+    *(volatile uint32_t *)ctx->chain_gave_up = 0u;
+    set_error(error, error_capacity, "a chained launch stopped waiting for the first linear's outputs after %u polls; "
+                                     "its results are not valid (without option \"chain\" the two linears run as two launches)",
+              ctx->chain_spin_limit);
+    return MI355Q_ERROR_RUNTIME;
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -79,6 +91,20 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "chain") == 0) {  // "1": gate|up-SiLU and the linear that reads it go out as one launch
+        ctx->chain_enabled = set && strcmp(value, "0") != 0;
+        return MI355Q_OK;
+    }
+    if (strcmp(name, "chain_spin_limit") == 0) {  // polls before a consumer wave of a chained launch stops waiting
+        unsigned limit = kChainSpinLimitDefault;
+        if (set && sscanf(value, "%u", &limit) != 1) return MI355Q_ERROR_INVALID;
+        ctx->chain_spin_limit = limit;
+        return MI355Q_OK;
+    }
+    if (strcmp(name, "chain_withhold") == 0) {  // "1": chained launches wait for a count they cannot reach
+        ctx->chain_withhold = set && strcmp(value, "0") != 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "in_kernel_slices") == 0) {  // "0": a second kernel adds the K slices
         ctx->columns_share_xcd = ctx->columns_probed && !(set && strcmp(value, "0") == 0);
         return MI355Q_OK;
@@ -98,6 +124,26 @@ int mi355q_context_set_option(mi355q_context *ctx, const char *name, const char 
     if (apply_option(ctx, name, value) != MI355Q_OK) {
         set_error(error, error_capacity, "context_set_option: unknown option or malformed value: %s=%s", name,
                   value ? value : "");
+        return MI355Q_ERROR_INVALID;
+    }
+    return MI355Q_OK;
+}
+
+int mi355q_context_get(mi355q_context *ctx, const char *name, uint64_t *value, char *error, size_t error_capacity)
+{
+    if (ctx == nullptr || name == nullptr || value == nullptr) {
+        set_error(error, error_capacity, "context_get: null argument");
+        return MI355Q_ERROR_INVALID;
+    }
+    if (strcmp(name, "chained_launches") == 0) {
+        *value = ctx->chain_total;
+    } else if (strcmp(name, "staging_bytes") == 0) {
+        *value = 0;
+        for (int slot = 0; slot < 6; ++slot) *value += ctx->stage_bytes[slot];
+    } else if (strcmp(name, "staging_generation") == 0) {
+        *value = ctx->stage_generation;
+    } else {
+        set_error(error, error_capacity, "context_get: unknown counter %s", name);
         return MI355Q_ERROR_INVALID;
     }
     return MI355Q_OK;
@@ -139,6 +185,11 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipEventCreate(&ctx->timer_stop);
     if (status == hipSuccess) status = hipMalloc((void **)&ctx->arrivals, kArrivalCounters * sizeof(uint32_t));
     if (status == hipSuccess) status = hipMemset(ctx->arrivals, 0, kArrivalCounters * sizeof(uint32_t));
+    if (status == hipSuccess) status = hipMalloc((void **)&ctx->chain_ready, kChainWords * sizeof(uint32_t));
+    if (status == hipSuccess) status = hipMemset(ctx->chain_ready, 0, kChainWords * sizeof(uint32_t));
+    if (status == hipSuccess) status = hipHostMalloc((void **)&ctx->chain_gave_up, sizeof(uint32_t), hipHostMallocDefault);
+    if (status == hipSuccess) *ctx->chain_gave_up = 0u;
+    ctx->chain_spin_limit = kChainSpinLimitDefault;
     if (status == hipSuccess) status = q4_stream_scratch_init(ctx);  // this device is current
     uint32_t xcds = 0;
     if (status == hipSuccess) status = probe_columns_share_xcd(ctx, &ctx->columns_share_xcd, &xcds);
@@ -148,6 +199,7 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     (void)apply_option(ctx, "q4_stream", getenv("MI355Q_Q4_STREAM"));
     (void)apply_option(ctx, "q4_gemm", getenv("MI355Q_Q4_GEMM"));
     (void)apply_option(ctx, "trace", getenv("MI355Q_TRACE"));
+    (void)apply_option(ctx, "chain", getenv("MI355Q_CHAIN"));
     if (status != hipSuccess) {
         int code = fail_hip(status, "context_create", error, error_capacity);
         mi355q_context_destroy(ctx);
@@ -169,6 +221,8 @@ void mi355q_context_destroy(mi355q_context *ctx)
         delete ctx->profile_events;
     }
     if (ctx->arrivals) (void)hipFree(ctx->arrivals);
+    if (ctx->chain_ready) (void)hipFree(ctx->chain_ready);
+    if (ctx->chain_gave_up) (void)hipHostFree(ctx->chain_gave_up);
     if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
     if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -202,7 +256,7 @@ int mi355q_sync(mi355q_context *ctx, char *error, size_t error_capacity)
         return MI355Q_ERROR_INVALID;
     }
     MI355Q_HIP(hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
-    return MI355Q_OK;
+    return chain_after_wait(ctx, error, error_capacity);
 }
 
 int mi355q_device_alloc(mi355q_context *ctx, size_t bytes, void **out, char *error,
@@ -256,7 +310,7 @@ int mi355q_download(mi355q_context *ctx, void *host_dst, const void *device_src,
     MI355Q_HIP(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, ctx->stream),
                "download");
     MI355Q_HIP(hipStreamSynchronize(ctx->stream), "download sync");
-    return MI355Q_OK;
+    return chain_after_wait(ctx, error, error_capacity);
 }
 
 int mi355q_timer_begin(mi355q_context *ctx, char *error, size_t error_capacity)
@@ -284,7 +338,7 @@ int mi355q_timer_end(mi355q_context *ctx, double *gpu_ms, char *error,
     MI355Q_HIP(hipEventElapsedTime(&ms, ctx->timer_start, ctx->timer_stop),
                "hipEventElapsedTime");
     *gpu_ms = (double)ms;
-    return MI355Q_OK;
+    return chain_after_wait(ctx, error, error_capacity);
 }
 
 int mi355q_profile_begin(mi355q_context *ctx, char *error, size_t error_capacity)
@@ -317,7 +371,7 @@ int mi355q_profile_end(mi355q_context *ctx, double *kernel_ms, uint64_t *launche
     }
     *kernel_ms = total;
     if (launches) *launches = ctx->profile_used / 2;
-    return MI355Q_OK;
+    return chain_after_wait(ctx, error, error_capacity);
 }
 
 int mi355q_profile_durations(mi355q_context *ctx, double *kernel_us, size_t capacity, size_t *count,
@@ -853,6 +907,47 @@ int mi355q_q4_linear_noalloc(mi355q_context *ctx, const mi355q_q4_weight *weight
     return MI355Q_OK;
 }
 
+// The arguments of two consecutive calls of a sequence as the launchers take them, when the pair
+// is the one that can go out as one launch: {gate, up} with MI355Q_FUSE_GATE_UP_SILU writing
+// fp16, then one weight whose activations are that output.  False: run them one by one (which
+// also reports whatever is wrong with them).
+static bool sequence_pair(mi355q_context *ctx, const mi355q_q4_call &first, const mi355q_q4_call &second,
+                          Q4LinearArgs &gate_up, Q4LinearArgs &down)
+{
+    if (first.flags != MI355Q_FUSE_GATE_UP_SILU || first.target_count != 2u || second.target_count != 1u) return false;
+    if ((second.flags & ~(uint32_t)MI355Q_RESIDUAL_IS_BIAS) != 0u) return false;
+    if (first.x == nullptr || second.x == nullptr || first.M == 0u || first.M != second.M) return false;
+    if (!dtype_valid(first.x_dtype) || first.y_dtype != MI355Q_F16 || second.x_dtype != MI355Q_F16 ||
+        !dtype_valid(second.y_dtype))
+        return false;
+    const mi355q_q4_target &gate = first.targets[0], &up = first.targets[1], &w = second.targets[0];
+    if (gate.weight == nullptr || up.weight == nullptr || w.weight == nullptr || gate.y == nullptr || w.y == nullptr)
+        return false;
+    if (gate.weight->ctx != ctx || up.weight->ctx != ctx || w.weight->ctx != ctx) return false;
+    if (gate.residual != nullptr || up.residual != nullptr) return false;
+    if (w.residual != nullptr && !dtype_valid(second.residual_dtype)) return false;
+    if (second.x != gate.y || ((uintptr_t)first.x & 15u) != 0u || ((uintptr_t)second.x & 15u) != 0u) return false;
+    memset(&gate_up, 0, sizeof gate_up);
+    gate_up.x = first.x;
+    gate_up.x_dtype = first.x_dtype;
+    gate_up.M = first.M;
+    gate_up.y_dtype = first.y_dtype;
+    gate_up.fuse_silu = true;
+    gate_up.count = 2;
+    gate_up.targets[0] = Q4Target{&gate.weight->dev, gate.y, nullptr};
+    gate_up.targets[1] = Q4Target{&up.weight->dev, up.y, nullptr};
+    memset(&down, 0, sizeof down);
+    down.x = second.x;
+    down.x_dtype = second.x_dtype;
+    down.M = second.M;
+    down.y_dtype = second.y_dtype;
+    down.residual_dtype = second.residual_dtype;
+    down.residual_is_bias = (second.flags & MI355Q_RESIDUAL_IS_BIAS) != 0u;
+    down.count = 1;
+    down.targets[0] = Q4Target{&w.weight->dev, w.y, w.residual};
+    return q4_chain_possible(ctx, gate_up, down);
+}
+
 int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, size_t count,
                               char *error, size_t error_capacity)
 {
@@ -864,6 +959,18 @@ int mi355q_q4_linear_sequence(mi355q_context *ctx, const mi355q_q4_call *calls, 
     for (size_t i = 0; i < count; ++i) {
         const mi355q_q4_call &c = calls[i];
         char inner[256] = "";
+        Q4LinearArgs gate_up, down;
+        if (i + 1 < count && sequence_pair(ctx, c, calls[i + 1], gate_up, down)) {
+            // gate|up with SiLU and the linear that reads its output: one launch for the two
+            MI355Q_HIP(hipSetDevice(ctx->device), "hipSetDevice");
+            int status = q4_chain_linear(ctx, gate_up, down, inner, sizeof inner);
+            if (status != MI355Q_OK) {
+                set_error(error, error_capacity, "calls %zu and %zu (one launch): %s", i, i + 1, inner);
+                return status;
+            }
+            ++i;
+            continue;
+        }
         const uint32_t own = c.flags & (MI355Q_RESIDUAL_IS_BIAS | MI355Q_FUSE_GATE_UP_SILU);
         int status = mi355q_q4_linear_multi(ctx, c.targets, c.target_count, c.x, c.x_dtype, c.M,
                                             c.y_dtype, c.residual_dtype, flags | own, inner, sizeof inner);

@@ -82,9 +82,28 @@ struct mi355q_context {
     // device address of the library's fixed scratch array on this context's device (for the
     // entry point that allocates nothing); every context on the device sees the same array
     unsigned char *fixed_scratch;
+    // Chained launches (gate|up with SiLU and down as one kernel, q4_chain.hip): one counter per
+    // 128-column step of the second linear's activations, counting announced tiles over all
+    // chained launches of the context (never reset: launch number n waits for 8 n), followed by
+    // the leaders' "slice complete" words (kChainWords in all); the word in
+    // pinned host memory that a consumer wave sets when it stops waiting; the polls after which
+    // it does.  Options "chain" = "1" (off unless asked for), "chain_spin_limit", and
+    // "chain_withhold" = "1" (the next launches wait for a count they cannot reach: the test of
+    // the bounded wait).
+    uint32_t *chain_ready;
+    uint32_t *chain_gave_up;
+    uint32_t chain_launches;  // chained launches the counters have seen since they were last zero
+    uint32_t chain_steps;     // steps (counters) those launches had; a pair with another count starts from zero again
+    uint64_t chain_total;     // chained launches of this context so far
+    uint32_t chain_spin_limit;
+    bool chain_enabled, chain_withhold;
+    bool chain_pending;  // a chained launch has been queued since the host last looked at chain_gave_up
 };
 namespace mi355q {
 constexpr uint32_t kArrivalCounters = 65536;
+constexpr uint32_t kChainCounters = 4096;            // steps of a chained pair's second linear (K <= 524288)
+constexpr uint32_t kChainWords = kChainCounters + 8u * 16u * 32u;  // + one cache line per (XCD, slice) leader
+constexpr uint32_t kChainSpinLimitDefault = 1u << 16;  // about a tenth of a second of polling
 }
 
 struct mi355q_q4_weight {
@@ -186,6 +205,14 @@ struct Q4LinearArgs {
 // device) and keeps it in the context; called by mi355q_context_create with that device current.
 hipError_t q4_stream_scratch_init(mi355q_context *ctx);
 int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity);
+// q4_chain.hip: may these two linears (gate|up with SiLU, then the linear that reads its output)
+// go out as one launch on this context, and the launch itself
+bool q4_chain_possible(const mi355q_context *ctx, const Q4LinearArgs &gate_up, const Q4LinearArgs &down);
+int q4_chain_linear(mi355q_context *ctx, const Q4LinearArgs &gate_up, const Q4LinearArgs &down, char *error,
+                    size_t error_capacity);
+// After the host has waited for the context's stream: status 1 (and the word cleared) if a
+// consumer wave of a chained launch stopped waiting since the last look.
+int chain_after_wait(mi355q_context *ctx, char *error, size_t error_capacity);
 // mi355q_q4_linear_multi with Q4LinearArgs::x_columns
 int q4_linear_multi_repeated(mi355q_context *ctx, const mi355q_q4_target *targets, uint32_t count, const void *x,
                              int x_dtype, uint32_t M, int y_dtype, int residual_dtype, uint32_t flags,

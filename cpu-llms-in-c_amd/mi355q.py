@@ -64,6 +64,7 @@ SIGNATURES = {
     "mi355q_context_destroy": (None, [_vp]),
     "mi355q_context_info": (_int, [_vp, _c.POINTER(DeviceInfo), *_err]),
     "mi355q_context_set_option": (_int, [_vp, _cp, _cp, *_err]),
+    "mi355q_context_get": (_int, [_vp, _cp, _c.POINTER(_u64), *_err]),
     "mi355q_sync": (_int, [_vp, *_err]),
     "mi355q_device_alloc": (_int, [_vp, _sz, _c.POINTER(_vp), *_err]),
     "mi355q_device_free": (_int, [_vp, _vp, *_err]),
@@ -251,6 +252,12 @@ class Context:
         """Experiment knob of this context (see mi355q_context_set_option); None clears it."""
         _call(self.lib.mi355q_context_set_option, self.handle, name.encode(),
               None if value is None else value.encode())
+
+    def get(self, name: str) -> int:
+        """A counter of the context: "chained_launches", "staging_bytes", "staging_generation"."""
+        value = ctypes.c_uint64()
+        _call(self.lib.mi355q_context_get, self.handle, name.encode(), ctypes.byref(value))
+        return int(value.value)
 
     def sync(self):
         _call(self.lib.mi355q_sync, self.handle)

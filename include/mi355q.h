@@ -126,9 +126,26 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *   "gemm_loads" = "plain"                      GEMM variant 7 built with ordinary weight loads
  *                                               (compiler-placed waits): the cross-check of the
  *                                               hand-scheduled kernel, same bits, slower
+ *   "chain" = "1"                               mi355q_q4_linear_sequence runs gate|up-SiLU and the
+ *                                               linear that reads its output as ONE launch (see there;
+ *                                               also MI355Q_CHAIN=1 in the environment).  Off by default:
+ *                                               measured on the 27B MLP it is 3 us slower than the two
+ *                                               launches at one row and level with them at two
+ *   "chain_spin_limit" = "N"                    polls after which a waiting wave of such a one-launch
+ *                                               pair gives up (the call that next waits for the
+ *                                               stream then returns status 1)
+ *   "chain_withhold" = "1"                      such launches wait for a count they cannot reach: the
+ *                                               test of that bounded wait
  * Unknown names and malformed values: status 2. */
 int mi355q_context_set_option(mi355q_context *ctx, const char *name, const char *value,
                               char *error, size_t error_capacity);
+/* Counters of one context, for tests and reports (no counterpart in the reference):
+ *   "chained_launches"    pairs of linears that went out as one launch (see mi355q_q4_linear_sequence)
+ *   "staging_bytes"       bytes of the context's growable staging buffers
+ *   "staging_generation"  how often a staging buffer has been reallocated
+ * Unknown names: status 2. */
+int mi355q_context_get(mi355q_context *ctx, const char *name, uint64_t *value,
+                       char *error, size_t error_capacity);
 /* Waits for everything queued on the context's stream
  * (the reference's waitUntilCompleted, qwen38_m3_decode.m:1701-1716). */
 int mi355q_sync(mi355q_context *ctx, char *error, size_t error_capacity);
@@ -383,7 +400,18 @@ int mi355q_q4_linear_multi(mi355q_context *ctx, const mi355q_q4_target *targets,
  * host call, all pointers on the device and nothing waited for — the way the
  * reference encodes every matvec of a forward pass into one command buffer
  * before committing it (qwen38_m3_decode.m:1614-1699).  Stops at the first
- * call that fails and reports its index in the message. */
+ * call that fails and reports its index in the message.
+ *
+ * With the context option "chain" = "1", two consecutive calls of the form  {gate, up} with
+ * MI355Q_FUSE_GATE_UP_SILU writing fp16, then one weight whose x is that output (fp16, same
+ * M <= 16; fp16 or bf16 x for the first) - the MLP of a decoder layer as the reference encodes
+ * it, mlp_gate_up then mlp_down with nothing between them (qwen38_m3_layer.m:314-336) - go
+ * out as ONE kernel launch when the launch shapes of the two linears allow it: the second
+ * linear's workgroups ask for their first weights at once and start multiplying when the
+ * first linear's outputs for their K slice are complete.  Same bits as the two launches.
+ * The wait is bounded; if a wave ever gives up, the next call that waits for the stream
+ * (mi355q_sync, mi355q_download, mi355q_timer_end, mi355q_profile_end) returns status 1 and
+ * the outputs are not valid.  Not used while a sequence is being recorded into a graph. */
 typedef struct {
     const void *x;
     uint32_t M;
