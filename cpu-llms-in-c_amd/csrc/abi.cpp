@@ -139,7 +139,7 @@ int mi355q_context_get(mi355q_context *ctx, const char *name, uint64_t *value, c
         *value = ctx->chain_total;
     } else if (strcmp(name, "staging_bytes") == 0) {
         *value = 0;
-        for (int slot = 0; slot < 6; ++slot) *value += ctx->stage_bytes[slot];
+        for (int slot = 0; slot < kStageSlots; ++slot) *value += ctx->stage_bytes[slot];
     } else if (strcmp(name, "staging_generation") == 0) {
         *value = ctx->stage_generation;
     } else {
@@ -214,7 +214,7 @@ void mi355q_context_destroy(mi355q_context *ctx)
     if (ctx == nullptr) return;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    for (int slot = 0; slot < 6; ++slot)
+    for (int slot = 0; slot < kStageSlots; ++slot)
         if (ctx->stage[slot]) (void)hipFree(ctx->stage[slot]);
     if (ctx->profile_events) {
         for (hipEvent_t event : *ctx->profile_events) (void)hipEventDestroy(event);

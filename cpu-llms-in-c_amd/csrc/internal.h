@@ -46,6 +46,9 @@ struct Q4Device {
 
 }  // namespace mi355q
 
+namespace mi355q {
+constexpr int kStageSlots = 7;
+}
 struct mi355q_context {
     int device;
     hipStream_t stream;
@@ -58,9 +61,10 @@ struct mi355q_context {
     std::vector<hipEvent_t> *profile_events;
     size_t profile_used;
     // staging: 0 host x, 1 host y, 2 host residual, 3 activations converted to fp16,
-    // 4 fp32 partial sums of a K-split GEMM, 5 the high-nibble half of an affine-Q8 linear
-    void *stage[6];
-    size_t stage_bytes[6];
+    // 4 fp32 partial sums of a K-split GEMM, 5 the high-nibble half of an affine-Q8 linear,
+    // 6 the fp32 outputs of a GEMM on converted activations, before their rows are finished
+    void *stage[mi355q::kStageSlots];
+    size_t stage_bytes[mi355q::kStageSlots];
     // bumped whenever a staging buffer is reallocated: recorded graphs hold the old
     // pointers and refuse to run once this has moved on
     uint64_t stage_generation;
@@ -205,6 +209,10 @@ struct Q4LinearArgs {
 // device) and keeps it in the context; called by mi355q_context_create with that device current.
 hipError_t q4_stream_scratch_init(mi355q_context *ctx);
 int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, size_t error_capacity);
+// bf16 / fp32 activations x[M][K] -> fp16 rows scaled by a power of two per row (bf16: M rows; fp32:
+// 2 M rows, value then rounding remainder) and row_scale[M], the factors that undo the scaling
+hipError_t q4_convert_x_launch(mi355q_context *ctx, const void *x, int x_dtype, _Float16 *out, float *row_scale,
+                               uint32_t M, uint32_t K);
 // q4_chain.hip: may these two linears (gate|up with SiLU, then the linear that reads its output)
 // go out as one launch on this context, and the launch itself
 bool q4_chain_possible(const mi355q_context *ctx, const Q4LinearArgs &gate_up, const Q4LinearArgs &down);

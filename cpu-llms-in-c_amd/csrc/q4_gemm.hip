@@ -82,16 +82,30 @@ __global__ void __launch_bounds__(256) q4_gemm_reduce_kernel(const GemmParams p)
     store_from_float(p.y, p.y_dtype, at, value);
 }
 
-// fp32 / bf16 activations are rounded to fp16 once per call (the matrix
-// instruction multiplies fp16 operands).
+// Activations that are not fp16 get the streaming kernel's treatment (q4_convert_x_launch): every
+// row scaled by a power of two into fp16's range, bf16 rows as one fp16 row, fp32 rows as two
+// (value, rounding remainder).  The matrix kernels then multiply those M or 2 M rows into an fp32
+// staging matrix, and this kernel finishes the outputs: the two rows of a pair added, the row's
+// scale taken out again, then residual and output type as in the matrix kernels' own epilogue.
+// (The reference's grouped linear keeps fp32 activations at any row count,
+// whisper_turbo_encoder.c:128-176; cpu_q4_dot_float, qwen38_m3_layer.m:375-393.)
 __global__ void __launch_bounds__(256)
-q4_gemm_convert_x_kernel(const void *__restrict__ x, int x_dtype, _Float16 *__restrict__ out,
-                         size_t count)
+q4_gemm_finish_kernel(const float *__restrict__ staged, const float *__restrict__ row_scale, int pair,
+                      void *__restrict__ y, int y_dtype, const void *__restrict__ residual, int residual_dtype,
+                      int residual_is_bias, uint32_t M, uint32_t N)
 {
-    const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (index >= count) return;
-    const float value = load_as_float(x, x_dtype, index), limit = 65504.0f;  // saturate, no infinities
-    out[index] = (_Float16)(value > limit ? limit : value < -limit ? -limit : value);
+    const size_t total = (size_t)M * N;
+    for (size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x; at < total; at += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t m = (uint32_t)(at / N), n = (uint32_t)(at % N);
+        float value;
+        if (pair)
+            value = staged[(size_t)(2u * m) * N + n] + staged[(size_t)(2u * m + 1u) * N + n];
+        else
+            value = staged[at];
+        value *= row_scale[m];
+        if (residual) value += load_as_float(residual, residual_dtype, residual_is_bias ? n : at);
+        store_from_float(y, y_dtype, at, value);
+    }
 }
 
 // The pipelined kernel's stage is larger than the 64 KiB a kernel gets without asking: the
@@ -141,26 +155,34 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         return MI355Q_ERROR_INVALID;
     }
     const uint32_t x_columns = a.x_columns ? a.x_columns : w.K;
-    if (a.x_dtype != MI355Q_F16) {
-        const size_t count = (size_t)a.M * x_columns;
-        int status = ensure_stage(ctx, 3, count * sizeof(_Float16), error, error_capacity);
+    // rows the matrix kernels see: M, or 2 M when fp32 activations go in as (value, remainder) pairs
+    const bool converted_x = a.x_dtype != MI355Q_F16, pair = a.x_dtype == MI355Q_F32;
+    const uint32_t rows = pair ? 2u * a.M : a.M;
+    const float *row_scale = nullptr;
+    if (converted_x) {
+        // [ the rows' inverse scales, padded to 256 bytes | rows * K fp16 ], then the fp32 staging matrix
+        const size_t scale_bytes = ((size_t)a.M * sizeof(float) + 255u) & ~(size_t)255u;
+        int status = ensure_stage(ctx, 3, scale_bytes + (size_t)rows * x_columns * sizeof(_Float16), error, error_capacity);
+        if (status == MI355Q_OK)
+            status = ensure_stage(ctx, 6, (size_t)rows * w.N * sizeof(float), error, error_capacity);
         if (status != MI355Q_OK) return status;
-        hipError_t converted =
-            launch(ctx, q4_gemm_convert_x_kernel, dim3((uint32_t)((count + 255u) / 256u)), dim3(256),
-                   0, a.x, a.x_dtype, (_Float16 *)ctx->stage[3], count);
+        float *const scales = (float *)ctx->stage[3];
+        _Float16 *const fp16_rows = (_Float16 *)((char *)ctx->stage[3] + scale_bytes);
+        hipError_t converted = q4_convert_x_launch(ctx, a.x, a.x_dtype, fp16_rows, scales, a.M, x_columns);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
-        p.x = (const _Float16 *)ctx->stage[3];
+        p.x = fp16_rows;
+        row_scale = scales;
     }
-    p.y = a.targets[target].y;
-    p.residual = a.targets[target].residual;
-    p.M = a.M;
+    p.y = converted_x ? ctx->stage[6] : a.targets[target].y;
+    p.residual = converted_x ? nullptr : a.targets[target].residual;
+    p.M = rows;
     p.N = w.N;
     p.K = x_columns;
     p.wrap_steps = a.x_columns ? a.x_columns / kStepColumns : 0xffffffffu;
     p.NT = w.NT;
     p.T = w.T;
-    p.y_dtype = a.y_dtype;
+    p.y_dtype = converted_x ? MI355Q_F32 : a.y_dtype;
     p.residual_dtype = a.residual_dtype;
     p.residual_is_bias = a.residual_is_bias;
     p.wide_stores = w.N % 4u == 0u && (uintptr_t)p.y % 16u == 0u;
@@ -198,13 +220,13 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     uint32_t best_splits = 1;
     double best_cost = 1e30;
     // the pipelined kernel addresses x with 32-bit byte offsets and whole 128-column steps
-    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)a.M * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
+    const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)rows * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
         if (v >= 6 && !pipe_ok) continue;
         const Variant &c = variants[v];
         const uint32_t tpb = 4u * c.ntw + c.extra;
         const uint32_t slots = cus * (uint32_t)c.resident;
-        const uint32_t m_blocks = (a.M + c.bm - 1) / c.bm;
+        const uint32_t m_blocks = (rows + c.bm - 1) / c.bm;
         const uint32_t n_blocks = (w.NT + tpb - 1) / tpb;
         for (uint32_t want = 1; want <= 8u && want * 8u <= w.T + 7u; ++want) {
             const uint32_t steps = (w.T + want - 1) / want;
@@ -234,7 +256,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
             else
                 cost = ((double)groups / slots + (groups % slots ? 0.31 : 0.0)) * c.resident * peak_us / c.shared;
             if (splits > 1)  // fp32 partials at 4.6 TB/s and the kernel that adds them
-                cost += (double)splits * a.M * (double)w.N * 4.0 / 4.63e6 + (v >= 6 ? 2.0 : 6.3);
+                cost += (double)splits * rows * (double)w.N * 4.0 / 4.63e6 + (v >= 6 ? 2.0 : 6.3);
             if (cost < best_cost) {
                 best_cost = cost;
                 best = v;
@@ -250,17 +272,17 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     }
     if (ctx->trace)
         fprintf(stderr, "mi355q: q4 gemm M=%u N=%u K=%u -> variant %d (BM=%d, %d tiles/wave%s), K split %u\n",
-                a.M, w.N, w.K, best, variants[best].bm, variants[best].ntw,
+                rows, w.N, w.K, best, variants[best].bm, variants[best].ntw,
                 variants[best].extra ? " +1" : "", best_splits);
     const Variant &chosen = variants[best];
     const uint32_t tpb = 4u * chosen.ntw + chosen.extra;
     p.tiles_per_block = tpb;
     const uint32_t n_blocks = (w.NT + tpb - 1) / tpb;
-    const uint32_t m_blocks = (a.M + chosen.bm - 1) / chosen.bm;
+    const uint32_t m_blocks = (rows + chosen.bm - 1) / chosen.bm;
     p.steps_per_split = (w.T + best_splits - 1) / best_splits;
     p.splits = (w.T + p.steps_per_split - 1) / p.steps_per_split;
     if (p.splits > 1u) {
-        const size_t bytes = (size_t)p.splits * a.M * w.N * sizeof(float);
+        const size_t bytes = (size_t)p.splits * rows * w.N * sizeof(float);
         int status = ensure_stage(ctx, 4, bytes, error, error_capacity);
         if (status != MI355Q_OK) return status;
         p.partials = (float *)ctx->stage[4];
@@ -281,7 +303,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);
     if (p.splits > 1u) {
-        const size_t total = (size_t)a.M * w.N;
+        const size_t total = (size_t)rows * w.N;
         if (p.wide_stores)
             launched = launch(ctx, q4_gemm_reduce_kernel<true>, dim3((uint32_t)((total / 4u + 255u) / 256u)),
                               dim3(256), 0, p);
@@ -290,6 +312,14 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
                               dim3(256), 0, p);
         if (launched != hipSuccess)
             return fail_hip(launched, "q4 gemm reduce launch", error, error_capacity);
+    }
+    if (converted_x) {
+        const size_t total = (size_t)a.M * w.N;
+        const uint32_t blocks = (uint32_t)((total + 255u) / 256u < 65536u ? (total + 255u) / 256u : 65536u);
+        launched = launch(ctx, q4_gemm_finish_kernel, dim3(blocks), dim3(256), 0, (const float *)ctx->stage[6], row_scale,
+                          pair ? 1 : 0, a.targets[target].y, a.y_dtype, a.targets[target].residual, a.residual_dtype,
+                          a.residual_is_bias ? 1 : 0, a.M, w.N);
+        if (launched != hipSuccess) return fail_hip(launched, "q4 gemm finish launch", error, error_capacity);
     }
     return MI355Q_OK;
 }

@@ -292,6 +292,12 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
     return shape;
 }
 
+hipError_t q4_convert_x_launch(mi355q_context *ctx, const void *x, int x_dtype, _Float16 *out, float *row_scale,
+                               uint32_t M, uint32_t K)
+{
+    return launch(ctx, q4_convert_x_kernel, dim3(M), dim3(kConvertThreads), 0, x, x_dtype, out, row_scale, M, K);
+}
+
 hipError_t zero_words_launch(mi355q_context *ctx, uint32_t *words, uint32_t count)
 {
     return launch(ctx, zero_words_kernel, dim3((count + 255u) / 256u), dim3(256), 0, words, count);
@@ -341,8 +347,7 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
         }
         float *const row_scale = (float *)area;
         _Float16 *const converted_x = (_Float16 *)(area + kRowScaleBytes);
-        hipError_t converted = launch(ctx, q4_convert_x_kernel, dim3(a.M), dim3(kConvertThreads), 0, a.x,
-                                      a.x_dtype, converted_x, row_scale, a.M, x_columns);
+        hipError_t converted = q4_convert_x_launch(ctx, a.x, a.x_dtype, converted_x, row_scale, a.M, x_columns);
         if (converted != hipSuccess)
             return fail_hip(converted, "activation conversion launch", error, error_capacity);
         p.x = converted_x;

@@ -346,6 +346,13 @@ int mi355q_q4_linear_rows(mi355q_context *ctx, const mi355q_q4_weight *weight,
  * [M][N] of residual_dtype.  The weight is evaluated as scale*q + bias without
  * rounding for M <= 16 (fp32 accumulation throughout); for larger M the weight
  * is rounded to fp16 before an fp16 matrix multiply with fp32 accumulation.
+ * Activations are never rounded to fp16 as they come: at every M, rows that are
+ * not fp16 are scaled by a power of two per row (undone in the epilogue), bf16
+ * rows then convert exactly and fp32 rows go through the matrix units as two
+ * fp16 rows, value and rounding remainder (about 22 significant bits) - the
+ * reference's grouped linear and its float-activation dots keep fp32
+ * activations at any row count (whisper_turbo_encoder.c:128-176;
+ * qwen38_m3_layer.m:375-393).
  * Replaces: cpu_row_dot / qwen38_q4_matvec (qwen38_m3.m:102-121;
  * qwen38_q4.metal:111-127), qwen38_q4_down_residual (qwen38_q4.metal:163-191),
  * the batched qwen38_prefill_q4_gemm_f16* family (qwen38_prefill.metal:144-248,

@@ -30,7 +30,7 @@ def run_case(engine, oracle, gpu, N, K, M, meta_kind, x_dtype, y_dtype, columns=
         x_ref, x_kind = x, oracle.X_BF16
     else:
         x = x32
-        x_ref, x_kind = x32.astype(np.float16), oracle.X_F16  # fp32 x is rounded to fp16 for M > 16
+        x_ref, x_kind = x32, oracle.X_F32  # fp32 rows go in as (value, remainder) pairs: not rounded
     res = engine.synth_normal_f32(seed + 2, 1.0, M * N).reshape(M, N) if residual else None
     weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, meta_kind)
     try:
@@ -118,6 +118,41 @@ def test_agrees_with_streaming_kernel_rows(engine, gpu):
 def test_dtypes_and_residual(engine, oracle, gpu, x_dtype, y_dtype):
     run_case(engine, oracle, gpu, 384, 512, 40, engine.META_F16_INTERLEAVED, getattr(engine, x_dtype),
              getattr(engine, y_dtype), residual=True)
+
+
+@pytest.mark.parametrize("forced", [None, "0,1", "3,2", "6,1", "7,2"])
+def test_activation_range(engine, oracle, gpu, force, forced):
+    """Activations far from fp16's range on the matrix-instruction path (64 rows): fp32 and bf16
+    rows of magnitude 1e4, 1e-3 and 1e-6 and rows with entries beyond 65504.  Rows that are not
+    fp16 are scaled by a power of two per row and fp32 rows go in as (value, remainder) pairs, so
+    the gate against the fp16-weight oracle on the caller's own x holds whatever the magnitude
+    (the reference keeps fp32 activations at any row count: whisper_turbo_encoder.c:128-176,
+    qwen38_m3_layer.m:375-393); with a residual and through a K split."""
+    N, K, M = 528, 1536, 64
+    if forced:
+        force("q4_gemm", forced)
+    quants, meta_a, meta_b = engine.synth_q4_affine(191, 0.02, N, K, engine.META_BF16_PLANES)
+    x = make_x(engine, 192, M, K).copy()
+    scales = np.ones(M, dtype=np.float32)
+    scales[0::4], scales[1::4], scales[2::4] = 1e4, 1e-3, 1e-6
+    x *= scales[:, None]
+    x[3, 5], x[3, 77], x[7, 1000] = np.float32(1e5), np.float32(-2.5e5), np.float32(7e4)
+    x_bf = bf16_bits(x).reshape(M, K)
+    res = engine.synth_normal_f32(193, 1.0, M * N).reshape(M, N) * scales[:, None]
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, engine.META_BF16_PLANES)
+    try:
+        print(f"gemm activation range case forced={forced}", flush=True)
+        y = gpu.q4_linear(weight, x, engine.F32, engine.F32, res, engine.F32)
+        y_bf = gpu.q4_linear(weight, x_bf, engine.BF16, engine.F32)
+    finally:
+        weight.destroy()
+    assert np.all(np.isfinite(y)) and np.all(np.isfinite(y_bf))
+    ref = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x, oracle.X_F32, M,
+                           weight_rounding=oracle.W_ROUND_F16) + res
+    assert q4_relative_error(y, ref) <= 1e-3
+    ref_bf = oracle.q4_linear(quants, meta_a, meta_b, engine.META_BF16_PLANES, N, K, x_bf, oracle.X_BF16, M,
+                              weight_rounding=oracle.W_ROUND_F16)
+    assert q4_relative_error(y_bf, ref_bf) <= 1e-3
 
 
 @pytest.mark.parametrize("forced", ["0,1", "1,2", "2,1", "3,1", "3,3", "4,1", "5,2", "6,1", "6,3", "7,1", "7,2", "8,1", "8,2"])
