@@ -115,6 +115,10 @@ def host_fields(oracle, threads, allowed):
         # a 2 GiB buffer: far beyond the last-level caches of any host
         "host_read_gib_per_s": {"threads_1": round(oracle.probe_read_gib_per_s(2 << 30, 1, 0.5), 2),
                                 "threads_%d" % threads: round(oracle.probe_read_gib_per_s(2 << 30, threads, 0.5), 2)},
+        "host_read_what": "sum over the threads of the bytes each reads per second from a 2 GiB buffer of 64-bit "
+                          "words (four accumulators per thread, 0.5 s); every pass a thread moves on to the share "
+                          "its neighbour read last, so over the passes each thread walks the whole buffer and no "
+                          "cache holds its working set: a DRAM figure",
     }
 
 
@@ -596,6 +600,112 @@ def bench_w8a8(engine, ctx, args):
     return 0
 
 
+# ---- configuration 1 ----------------------------------------------------------------------------
+
+def sym128_records(weights):
+    """fp32 [N][K] -> the symmetric group-128 records of compiler/q4_image.py as the C runtimes read
+    them (qwen35_task.c:286-303,426-450): per (row, 128 columns) a bf16 scale and 64 code bytes, element
+    j in byte j/2, even j in the low nibble, a two's complement value in [-8, 7]."""
+    N, K = weights.shape
+    blocks = weights.reshape(N, K // 128, 128)
+    scale = np.maximum(-blocks.min(axis=-1) / np.float32(8.0), blocks.max(axis=-1) / np.float32(7.0))
+    scale[scale == 0] = np.float32(1.0)
+    bits = scale.astype(np.float32).view(np.uint32).astype(np.uint64)
+    bf16 = (((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+    scale = (bf16.astype(np.uint32) << 16).view(np.float32)
+    nibbles = (np.clip(np.rint(blocks / scale[..., None]), -8, 7).astype(np.int16) & 0xF).astype(np.uint8)
+    records = np.empty((N, K // 128, 66), dtype=np.uint8)
+    records[..., :2] = bf16.view(np.uint8).reshape(N, K // 128, 2)
+    records[..., 2:] = nibbles[..., 0::2] | (nibbles[..., 1::2] << 4)
+    return np.ascontiguousarray(records).reshape(-1)
+
+
+def measure_config1(engine, ctx, with_cpu=True, copies=600, steps=1200):
+    """BASELINE configuration 1: the 0.8B-scale linear K=1024, N=3584 at M=1, affine-Q4 g64 with fp16
+    scale+bias, fp16 x and y (2,073,600 algorithmic bytes a call), rotating over `copies` prepared
+    copies; and the same shape in the symmetric group-128 format with fp32 x and y, which is what the
+    reference's portable runtime runs on CPU (q4_gemv, qwen35_task.c:318-362)."""
+    (name, N, K), = CONFIG1
+    work = LayerWorkload(engine, ctx, CONFIG1, copies, engine.META_F16_INTERLEAVED, 1)
+    r = measure_layer(ctx, work, 1, steps, 100, 20.0)
+    out = {
+        "workload": "affine-Q4 g64 GEMV K=%d N=%d M=1, fp16 scale+bias, fp16 x and y" % (K, N),
+        "gb_per_s": round(r["value"], 1), "steps": steps, "weight_copies_rotated": copies,
+        "rotated_bytes": r["step_bytes"] * copies, "kernel_us_per_launch_p50": round(r["kernel_us_per_step"][1], 2),
+        "wall_us_per_call": round(r["wall"] / steps * 1e6, 2),
+        "roofline": {"bound": "hbm", "achieved": round(r["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4), "kernel": "q4_stream_kernel",
+                     "avg_kernel_us": round(r["avg_kernel_us"], 3),
+                     "algorithmic_bytes_per_launch": round(r["bytes_per_launch"], 1)},
+    }
+    # the same shape as symmetric group-128 records: prepared once per copy, fp32 in and out
+    weights32 = engine.synth_normal_f32(4242, 0.02, N * K).reshape(N, K)
+    records = sym128_records(weights32)
+    x32 = engine.synth_normal_f32(4243, 1.0, K)
+    sym_copies = 64
+    sym = [ctx.sym128_prepare(records, N, K) for _ in range(sym_copies)]
+    x_ptr, y_ptr = ctx.to_device(x32), ctx.alloc(N * 4)
+    state = {"i": 0}
+
+    def run_steps(n):
+        for _ in range(n):
+            ctx.q4_linear_device(sym[state["i"] % sym_copies], x_ptr, engine.F32, 1, y_ptr, engine.F32)
+            state["i"] += 1
+
+    timed = time_steps(ctx, run_steps, 400, 40, 10.0, preheat_batch=100)
+    out["sym128_m1"] = {"workload": "symmetric Q4 g128 records (66 bytes a group), fp32 x and y, same shape",
+                        "record_bytes": int(records.size), "launches_per_call": timed["launches"] // 400,
+                        "kernel_us_per_call": round(timed["kernel_ms"] * 1e3 / 400, 2),
+                        "wall_us_per_call": round(timed["wall"] / 400 * 1e6, 2)}
+    if with_cpu:
+        import oracle  # test infrastructure, used here only as the timed CPU baseline
+        threads, allowed = host_threads()
+        quants, meta_a, meta_b = work.host[name]
+        x16 = work.host[("x", K)][:1]
+
+        def median_seconds(call, repeats=200):
+            call()
+            times = []
+            for _ in range(repeats):
+                t0 = time.perf_counter()
+                call()
+                times.append(time.perf_counter() - t0)
+            return sorted(times)[len(times) // 2]
+
+        affine = lambda n: oracle.q4_linear(quants, meta_a, meta_b, engine.META_F16_INTERLEAVED, N, K, x16, oracle.X_F16,
+                                            1, oracle.W_EXACT, oracle.ACC_F32_SEQUENTIAL, threads=n)
+        seconds, seconds4 = median_seconds(lambda: affine(threads)), median_seconds(lambda: affine(4))
+        bytes_call = q4_bytes(N, K, 1)
+        out["cpu_baseline"] = {
+            "value": round(bytes_call / seconds / 1e9, 3), "value_at_4_threads": round(bytes_call / seconds4 / 1e9, 3),
+            "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "200 calls (median), oracle restatement of cpu_row_dot, OpenMP static over rows, %.1f us a call"
+                      % (seconds * 1e6)}
+        sym_bytes = records.size + K * 4 + N * 4
+        restated = median_seconds(lambda: oracle.sym128_gemv(records, 0, N, K, x32, threads=threads))
+        column = {"value": round(sym_bytes / restated / 1e9, 3), "unit": "GB/s of the record image", "cores": threads,
+                  "kind": "port", "us_per_call": round(restated * 1e6, 1),
+                  "sample": "200 calls (median), oracle restatement of q4_gemv (qwen35_task.c:318-362), OpenMP static "
+                            "over rows"}
+        reference = oracle.ref_qwen35()
+        if reference is not None:  # the reference's own q4_gemv compiled from where it lies (oracle/_ref)
+            y = np.empty(N, dtype=np.float32)
+            own = median_seconds(lambda: reference.ref_qwen35_q4_gemv(records.ctypes.data, 0, N, K, x32.ctypes.data,
+                                                                      y.ctypes.data))
+            column["reference_build"] = {
+                "value": round(sym_bytes / own / 1e9, 3), "unit": "GB/s of the record image", "kind": "reference",
+                "us_per_call": round(own * 1e6, 1), "cores": os.environ.get("OMP_NUM_THREADS") or allowed,
+                "sample": "200 calls (median) of the reference's own q4_gemv (its OpenMP pragma, the process's "
+                          "thread count)"}
+        out["sym128_m1"]["cpu_baseline"] = column
+    for pointer in (x_ptr, y_ptr):
+        ctx.free(pointer)
+    for weight in sym:
+        weight.destroy()
+    work.destroy()
+    return out
+
+
 # ---- the secondary figures of the default line --------------------------------------------------
 
 def secondary_figures(engine, ctx, work, args):
@@ -614,13 +724,32 @@ def secondary_figures(engine, ctx, work, args):
             "kernel_us_per_step_p50": round(r["kernel_us_per_step"][1], 2),
             "kernel_us_per_launch_p50_in_launch_order": r["launch_p50"],
         }
+    # decode-identical verify (option "batch_invariant"): every row count takes the one-row launch's
+    # waves and K slices, so a row's bits do not depend on the batch; what that costs per row count
+    ctx.set_option("batch_invariant", "1")
+    invariant = {}
+    for M in (1, 2, 4, 8):
+        r = measure_layer(ctx, work, M, 100, 10, 10.0)
+        invariant["m%d" % M] = {"kernel_us_per_step_p50": round(r["kernel_us_per_step"][1], 2),
+                                "kernel_us_per_launch_p50_in_launch_order": r["launch_p50"],
+                                "hbm_frac_of_kernel_time": round(r["achieved"] / HBM_PEAK_GBPS, 4)}
+    ctx.set_option("batch_invariant", None)
+    out["verify_batch_invariant"] = {
+        "what": "the layer with option batch_invariant = 1: row m of an M-row call equals the one-row call on "
+                "x[m] bit for bit (compare kernel_us_per_step_p50 with verify_m* and the headline)",
+        **invariant}
     # prefill: the MLP weights of the layer (every copy), M = 512
     mlp = [[copy[4], copy[5], copy[6]] for copy in work.weights]
     host = {name: work.host[name] for name, _, _ in PREFILL}
     p = measure_prefill(engine, ctx, 512, 30, 5, 50.0, weights=mlp, host=host, with_cpu=not args.no_cpu)
     out["prefill_m512"] = {"tflops": p["tflops"], "percent_of_f16_peak": p["percent_of_f16_peak"],
                            "steps": 30, "warmup": 5, "linears_per_step": 3,
-                           "algorithmic_flops_per_step": p["step_flops"], "roofline": p["roofline"]}
+                           "algorithmic_flops_per_step": p["step_flops"], "roofline": p["roofline"],
+                           # what the matrix instruction sustains here from registers (power-limited clock):
+                           # alone, and with two or three packed-fp16 vector instructions between two of them
+                           "measured_mfma_tflops": {"alone": round(ctx.probe_mfma_rate(0), 1),
+                                                    "with_2_valu": round(ctx.probe_mfma_rate(2), 1),
+                                                    "with_3_valu": round(ctx.probe_mfma_rate(3), 1)}}
     if "cpu_baseline" in p:
         out["prefill_m512"]["cpu_baseline"] = p["cpu_baseline"]
     # the same three linears at M = 2048 (the shape divides evenly over the compute units from there on)
@@ -637,6 +766,7 @@ def secondary_figures(engine, ctx, work, args):
         out["w8a8_m64_k1024_n4096"]["bit_exact_vs_oracle"] = w["bit_exact_vs_oracle"]
         out["w8a8_m64_k1024_n4096"]["cpu_baseline"] = w["cpu_baseline"]
     out.update(measure_q8_affine(engine, ctx))
+    out["config1_m1"] = measure_config1(engine, ctx, with_cpu=not args.no_cpu)
     return out
 
 

@@ -91,6 +91,10 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "batch_invariant") == 0) {
+        ctx->batch_invariant = set && strcmp(value, "0") != 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "chain") == 0) {  // "1": gate|up-SiLU and the linear that reads it go out as one launch
         ctx->chain_enabled = set && strcmp(value, "0") != 0;
         return MI355Q_OK;

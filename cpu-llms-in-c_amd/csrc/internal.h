@@ -80,6 +80,9 @@ struct mi355q_context {
     int force_stream[4];  // tiles, depth, waves, slices (0 = not forced); [0] == 0: no forcing
     int force_gemm[2];    // kernel variant, K splits; [1] == 0: no forcing
     bool trace;           // print the chosen decomposition of every launch to stderr
+    // option "batch_invariant" = "1": streaming launches of up to eight activation rows take the
+    // waves and K slices of the one-row launch, so that a row's result does not depend on the batch
+    bool batch_invariant;
     bool gemm_plain_loads;  // option "gemm_loads" = "plain": the 17-tile GEMM shape with compiler-managed weight loads
     int w8a8_tiles;       // option "w8a8" = "1" .. "4": tiles per W8A8 workgroup (0: chosen by the launch)
     bool lds_raised[16];  // q4_gemm_pipe_kernel instantiations whose dynamic LDS limit has been raised

@@ -50,9 +50,9 @@ static hipError_t chain_launch_one(mi355q_context *ctx, dim3 grid, size_t lds, c
 static bool chain_shapes(const mi355q_context *ctx, const Q4LinearArgs &gate_up, const Q4LinearArgs &down, int mp)
 {
     const Q4Device &gate = *gate_up.targets[0].w, &w = *down.targets[0].w;
-    StreamShape a = choose_shape(ctx, 2u * gate.NT, gate.T, mp);
+    StreamShape a = choose_shape(ctx, 2u * gate.NT, gate.T, mp, true);
     if (a.tb != 2 && a.tb != 4) a.tb = 2;  // as q4_stream_plan pairs gate and up tiles
-    const StreamShape b = choose_shape(ctx, w.NT, w.T, mp);
+    const StreamShape b = choose_shape(ctx, w.NT, w.T, mp, false);
     return a.tb == 2 && a.depth == 2 && a.waves == 4 && a.slices == 1u && b.tb == (mp <= 2 ? 1 : 2) && b.depth == 2 &&
            b.waves == 4;
 }
@@ -71,7 +71,7 @@ bool q4_chain_possible(const mi355q_context *ctx, const Q4LinearArgs &gate_up, c
     while ((uint32_t)mp < gate_up.M) mp *= 2;
     if (!chain_shapes(ctx, gate_up, down, mp)) return false;
     // K slices of the consumers are added inside the kernel (a second kernel would be a second launch)
-    const StreamShape b = choose_shape(ctx, w.NT, w.T, mp);
+    const StreamShape b = choose_shape(ctx, w.NT, w.T, mp, false);
     return b.slices <= kChainMaxSlices && (b.slices <= 1u || ctx->columns_share_xcd);
 }
 

@@ -236,11 +236,25 @@ static void choose_cuts(StreamShape &shape, uint32_t T, uint32_t slices)
     shape.slices = (T + shape.slice_steps - 1) / shape.slice_steps;
 }
 
-StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp)
+StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp, bool fused)
 {
     StreamShape shape;
-    shape.mp = mp;
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    if (ctx->batch_invariant && mp > 1 && mp <= 8 && ctx->force_stream[0] <= 0) {
+        // Option "batch_invariant": which steps a wave takes, the order in which the waves' sums and
+        // the K slices are added - everything the bits of an output depend on - follows from the
+        // waves per workgroup and the slices, so both are those of the one-row launch of the same
+        // weights (held to eight waves, four for a fused gate|up pair, so that they fit the LDS of
+        // eight rows; the one-row launch in this mode is held to the same).  Row m of the result
+        // is then bit for bit the one-row call on x[m].  The tiles per workgroup may differ (tiles
+        // do not meet): two where the activations of four or more rows are worth sharing.
+        shape = choose_shape(ctx, NT_total, T, 1, fused);
+        shape.mp = mp;
+        shape.tb = mp >= 4 && NT_total >= cus ? 2 : mp >= 4 ? 1 : shape.tb;
+        while (shape.tb > 1 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u) shape.tb /= 2;
+        return shape;
+    }
+    shape.mp = mp;
     shape.tb = 1;
     shape.depth = 2;
     uint32_t slices = 1;
@@ -286,6 +300,10 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         if (ctx->force_stream[3] >= 1) slices = (uint32_t)ctx->force_stream[3];
     }
     choose_cuts(shape, T, slices);
+    if (ctx->batch_invariant && mp == 1 && ctx->force_stream[0] <= 0) {
+        const int most = fused ? 4 : 8;
+        if (shape.waves > most) shape.waves = most;
+    }
     while (shape.waves > 2 && (uint32_t)shape.waves > shape.slice_steps) shape.waves /= 2;
     while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
         shape.waves /= 2;
@@ -363,7 +381,7 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
     uint32_t tiles = 0;
     for (uint32_t t = 0; t < a.count; ++t)
         tiles += subset ? (a.row_count + kTileRows - 1) / kTileRows : a.targets[t].w->NT;
-    StreamShape shape = choose_shape(ctx, tiles, first.T, mp);
+    StreamShape shape = choose_shape(ctx, tiles, first.T, mp, a.fuse_silu);
     if (a.fuse_silu && shape.tb != 2 && shape.tb != 4) shape.tb = 2;  // gate and up tiles pair up
     if (shape.tb > 1 && shape.waves > 8) shape.waves = 8;  // sixteen waves exist for single tiles only
     while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)

@@ -25,8 +25,9 @@ struct StreamPlan {
 
 // dynamic LDS of a workgroup of the streaming kernel
 size_t stream_lds_bytes(int mp, int tb, int depth, int waves);
-// the launch shape for NT_total tiles of T steps and mp (a power of two) activation rows
-StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp);
+// the launch shape for NT_total tiles of T steps and mp (a power of two) activation rows;
+// fused: a gate|up pair whose workgroups take a tile of each
+StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp, bool fused);
 // Checks the arguments of a streaming linear, converts activations that are not fp16 (a kernel
 // on the context's stream), sizes the staging buffers and fills in the plan.  Nothing of the
 // linear itself has been launched when it returns.

@@ -126,6 +126,13 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *   "gemm_loads" = "plain"                      GEMM variant 7 built with ordinary weight loads
  *                                               (compiler-placed waits): the cross-check of the
  *                                               hand-scheduled kernel, same bits, slower
+ *   "batch_invariant" = "1"                     decode-identical verify: for up to eight activation
+ *                                               rows (four of fp32) row m of y is bit for bit what the
+ *                                               one-row call on x[m] gives, as the reference's exact
+ *                                               batched kernels guarantee (qwen38_prefill.metal:5-9,
+ *                                               142-248; tests/qwen38_m3_prefill_parity_test.c:115-199):
+ *                                               the launch takes the waves and K slices of the one-row
+ *                                               launch instead of the fastest ones for its row count
  *   "chain" = "1"                               mi355q_q4_linear_sequence runs gate|up-SiLU and the
  *                                               linear that reads its output as ONE launch (see there;
  *                                               also MI355Q_CHAIN=1 in the environment).  Off by default:

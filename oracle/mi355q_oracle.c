@@ -591,7 +591,10 @@ void orc_recipe_qwen38_weights(uint32_t seed, size_t group_count, uint8_t *quant
  * run_read_benchmark, tools/target_probe.c:60-160): every thread sums its own share of a
  * buffer of 64-bit words with four independent accumulators, pass after pass, until
  * `seconds` have gone by; the figure is bytes read / the longest thread's time, in GiB/s.
- * The buffer (bytes, at least 64 MiB to get past the caches) is written once first.
+ * The buffer (bytes, at least 64 MiB to get past the caches) is written once first.  From pass
+ * to pass a thread moves on to the next thread's share, so each thread walks the whole buffer
+ * and what a cache kept of the last pass is of no use to it: the figure is a DRAM figure even
+ * where one share would fit a last-level cache.
  * Not part of the path: context for the cpu_baseline figures.  Returns 0 on failure. */
 double orc_probe_read_gib_per_s(size_t bytes, int threads, double seconds, uint64_t *checksum_out)
 {
@@ -607,13 +610,14 @@ double orc_probe_read_gib_per_s(size_t bytes, int threads, double seconds, uint6
     {
         const int index = omp_get_thread_num(), count = omp_get_num_threads();
         const size_t share = words / (size_t)count;
-        const uint64_t *data = buffer + (size_t)index * share;
-        const size_t mine = (index == count - 1 ? words - (size_t)index * share : share) & ~(size_t)3;
+        const size_t mine = share & ~(size_t)3;
         uint64_t sum0 = 0, sum1 = 0, sum2 = 0, sum3 = 0, read = 0;
+        size_t pass = 0;
 #pragma omp barrier
         const double start = omp_get_wtime();
         double now;
         do {
+            const uint64_t *data = buffer + (((size_t)index + pass++) % (size_t)count) * share;
             for (size_t i = 0; i < mine; i += 4) {
                 sum0 += data[i];
                 sum1 += data[i + 1];
