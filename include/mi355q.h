@@ -370,9 +370,11 @@ int mi355q_q4_linear(mi355q_context *ctx, const mi355q_q4_weight *weight,
                      const void *residual, int residual_dtype,
                      uint32_t flags, char *error, size_t error_capacity);
 
-/* mi355q_q4_linear for callers that cannot allocate device memory while they run: code
- * under HIP graph capture, tight serving loops, harnesses that forbid it.  No counterpart in
- * the reference.  Same result as mi355q_q4_linear, bit for bit (same kernels, same launch
+/* mi355q_q4_linear for callers that cannot allocate device memory while they run: tight
+ * serving loops, harnesses that forbid hipMalloc, hosts whose allocator must stay quiet
+ * between two points (the call runs on the context's own stream, so it is not a node a
+ * caller's graph capture could record; mi355q_q4_sequence_record is the graph path).  No
+ * counterpart in the reference.  Same result as mi355q_q4_linear, bit for bit (same kernels, same launch
  * shapes), for 1..16 activation rows (8 of fp32); x, y and residual are DEVICE pointers
  * (the *_DEVICE flags are implied), x 16-byte aligned.  It calls no hipMalloc / hipFree
  * and no other allocating routine: what the ordinary call keeps in growable staging

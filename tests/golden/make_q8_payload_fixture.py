@@ -5,8 +5,13 @@ The quantizer is `q8_payload` (compiler/compile_minimindo_sensevoice_image.py:38
 on torch, with nothing in the reference's tests or C sources that fixes its rounding
 (float32 row divided by a Python double, torch.round, the double scale packed as "<f").  No
 closed form or other fixture pins those choices, so this script imports that one function from
-the reference tree and records what it returns.  Run it in the build container only (the
-reference tree exists only there); the tests read the committed .npz and never the reference.
+the reference tree and records what it returns.
+
+THIS SCRIPT EXECUTES REFERENCE CODE: importing the packer module runs that file's top-level
+statements and its imports (torch among them).  Run it only in the sandboxed build container,
+where the reference tree lives and nothing of value is within reach; never on a workstation
+or the GPU box.  The tests read the committed .npz (numpy.load, allow_pickle=False) and never
+the reference.
 
     python tests/golden/make_q8_payload_fixture.py
 """

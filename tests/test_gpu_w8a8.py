@@ -37,30 +37,65 @@ def test_config5(engine, oracle, gpu):
                                    (130, 2048, 512), (64, 1024, 4100), (5, 1024, 40), (17, 3072, 1000),
                                    (33, 1024, 16400), (64, 2048, 12304)])
 def test_shapes(engine, oracle, gpu, M, K, N):
-    """A workgroup takes one to four tiles by the launch's tile count (3, 63, 1025 and 769 tiles
-    among these), its last tiles may not exist, K of one to three 1024-column rounds and ragged
-    ones, row counts that end inside a fragment."""
+    """Tile counts of 1 to 1025 (the launch takes one tile per workgroup unless option "w8a8" asks
+    for more: test_tiles_per_workgroup_give_the_same_bits), K of one to three 1024-column rounds
+    and ragged ones, row counts that end inside a fragment."""
     check(engine, oracle, gpu, M, K, N, 7 + M, bias=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("M,K,N,channel_major", [(64, 1024, 4096, False), (21, 2048, 530, True)])
-def test_both_kernels_give_the_same_bits(engine, gpu, force, M, K, N, channel_major):
-    """Several tiles per workgroup and one tile per workgroup on the same call."""
+@pytest.mark.parametrize("M,K,N,channel_major", [(64, 1024, 4096, False), (21, 2048, 530, True),
+                                                 (9, 1024, 4100, False), (40, 560, 4100, True)])
+def test_tiles_per_workgroup_give_the_same_bits(engine, oracle, gpu, force, M, K, N, channel_major):
+    """One to four weight tiles per workgroup (option "w8a8"; the default launch takes one): the
+    multi-tile kernels share the activation registers between their tiles and keep one partial sum
+    area per tile in LDS.  Every setting gives the one-tile launch's bits and the oracle's; N = 4100
+    is 257 tiles, so with two, three and four tiles a workgroup the last workgroup's tiles partly
+    do not exist; M = 9, 21 and 40 fall into the one-, two- and four-fragment row blocks."""
     x = engine.synth_normal_f32(5, 1.0, M * K).reshape(M, K)
     rows = engine.synth_w8_rows(6, 0.02, N, K)
     bias = engine.synth_normal_f32(7, 1.0, N)
     q, scales = gpu.quantize_i8(x)
     weight = gpu.w8a8_prepare(rows, N, K)
+    results = {}
     try:
-        print(f"w8a8 both kernels M={M} K={K} N={N} channel_major={channel_major}", flush=True)
-        shared = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
-        force("w8a8", "1")
-        per_tile = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
+        print(f"w8a8 tiles per workgroup M={M} K={K} N={N} channel_major={channel_major}", flush=True)
+        results["default"] = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
+        for tiles in ("1", "2", "3", "4"):
+            force("w8a8", tiles)
+            results[tiles] = gpu.w8a8_linear(weight, N, q, scales, bias, channel_major=channel_major)
     finally:
         gpu.w8a8_destroy(weight)
-    assert shared[1].tobytes() == per_tile[1].tobytes()
-    assert np.array_equal(shared[0].view(np.uint32), per_tile[0].view(np.uint32))
-    assert np.any(shared[1] != 0)
+    out_ref, acc_ref = oracle.w8a8_linear(rows, N, K, q, scales, bias)
+    if channel_major:
+        out_ref = oracle.w8a8_conv(rows, N, K, q, scales, bias)
+    assert np.any(acc_ref != 0)
+    for name, (out, acc) in results.items():
+        assert acc.tobytes() == acc_ref.tobytes(), name
+        assert np.array_equal(out.view(np.uint32), out_ref.view(np.uint32)), name
+
+
+@pytest.mark.parametrize("tiles", ["2", "3", "4"])
+def test_shared_activation_launch_with_several_tiles_per_workgroup(engine, oracle, gpu, force, tiles):
+    """Three weights in one launch (workgroup ranges map to weights) with several tiles per
+    workgroup: the first workgroup of a weight starts at that weight's first tile whatever the
+    tile counts in front of it (here 257, 7 and 33 tiles)."""
+    M, K, widths = 23, 560, (4100, 100, 528)
+    x = engine.synth_normal_f32(171, 1.0, M * K).reshape(M, K)
+    q, scales = oracle.quantize_i8(x)
+    rows = [engine.synth_w8_rows(180 + i, 0.02, N, K) for i, N in enumerate(widths)]
+    biases = [engine.synth_normal_f32(190 + i, 1.0, N) for i, N in enumerate(widths)]
+    weights = [gpu.w8a8_prepare(r, N, K) for r, N in zip(rows, widths)]
+    try:
+        print(f"w8a8 shared activation, {tiles} tiles per workgroup", flush=True)
+        force("w8a8", tiles)
+        results = gpu.w8a8_linear_multi(weights, widths, q, scales, biases)
+    finally:
+        for weight in weights:
+            gpu.w8a8_destroy(weight)
+    for i, N in enumerate(widths):
+        out_ref, acc_ref = oracle.w8a8_linear(rows[i], N, K, q, scales, biases[i])
+        assert results[i][1].tobytes() == acc_ref.tobytes()
+        assert np.array_equal(results[i][0].view(np.uint32), out_ref.view(np.uint32))
 
 
 def test_reference_golden_vectors(engine, gpu):

@@ -2,7 +2,8 @@
 through the C ABI, bit for bit: same kernels and launch shapes, but converted activations,
 slice partial sums and arrival counters live in the library's fixed device array.
 
-Two calls in a row on each weight, the second with a smaller input, so that what the first
+The non-allocating call runs first on a fresh context and must leave the context's staging
+buffers as they were (none).  Two calls in a row on each weight, the second with a smaller input, so that what the first
 call left in the shared array (larger partial sums, counters, converted rows) must not leak
 into the second.  Runs alone in a fresh process and after the other tests alike: it makes its
 own context and cares nothing for what ran before.
@@ -48,9 +49,15 @@ def test_noalloc_matches_ordinary_call_bitwise(engine, oracle, name, N, K, x_dty
             pointers += [p for p in (x_ptr, y_ptr, z_ptr, r_ptr) if p]
             for pointer in (y_ptr, z_ptr):
                 ctx.upload(pointer, np.full((M, N), np.nan, dtype=np.float32))
+            # the non-allocating call first, on a context whose staging buffers the ordinary call has
+            # not yet grown for this size: it must not touch them (nothing allocated, nothing freed)
+            staging = (ctx.get("staging_bytes"), ctx.get("staging_generation"))
+            ctx.q4_linear_noalloc(weight, x_ptr, x_dtype, M, z_ptr, engine.F32, r_ptr, engine.F32)
+            assert (ctx.get("staging_bytes"), ctx.get("staging_generation")) == staging
+            if call == 0:
+                assert staging == (0, 0)  # a fresh context: the library has allocated no staging at all
             ctx.q4_linear_device(weight, x_ptr, x_dtype, M, y_ptr, engine.F32, r_ptr, engine.F32,
                                  asynchronous=False)
-            ctx.q4_linear_noalloc(weight, x_ptr, x_dtype, M, z_ptr, engine.F32, r_ptr, engine.F32)
             expect = ctx.download(y_ptr, (M, N), np.float32)
             got = ctx.download(z_ptr, (M, N), np.float32)
             assert np.array_equal(got.view(np.uint32), expect.view(np.uint32)), f"call {call} (M={M})"
