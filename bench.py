@@ -53,8 +53,9 @@ sys.path.insert(0, str(ROOT / "oracle"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X datasheet: 8 TB/s HBM3E
 # HBM bytes moved per algorithmic byte by the streaming kernel on the default workload: FETCH_SIZE and
-# WRITE_SIZE of rocprofv3 --pmc, scaled by a plain 2 GiB read/fill in the same runs
-# (profiles/q4_stream_kernel_layer_m1.md); a counter reading, not something this script can measure
+# WRITE_SIZE of rocprofv3 --pmc, scaled by a plain read/fill of known size in the same runs
+# (profiles/q4_stream_kernel_layer_m1.md, the section on the current library: 193,100,800 HBM bytes a
+# step against 191,897,600 algorithmic); a counter reading, not something this script can measure
 MEASURED_TRAFFIC_RATIO_LAYER_M1 = 1.006
 F16_MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 matrix instructions
 I8_MFMA_PEAK_TOPS = 5000.0  # dense int8 matrix instructions
@@ -203,7 +204,9 @@ class LayerWorkload:
 
     def calls(self, M, fuse=True, silu=False):
         """One call array per copy: linears that read the same activations go out as one launch
-        (q|k|v, gate|up); rows 0..M-1 of the activations."""
+        (q|k|v, gate|up); rows 0..M-1 of the activations.  silu: the gate|up launch writes
+        h = silu(gate . x) * (up . x) into gate's output buffer and down_proj reads that h (the MLP
+        as a layer runs it) instead of its own synthetic activations."""
         engine, out = self.engine, []
         for copy in range(self.copies):
             groups = []
@@ -213,11 +216,13 @@ class LayerWorkload:
                 if share:
                     groups[-1][0].append(target)
                 else:
-                    groups.append(([target], K))
-            out.append(engine.make_calls([
-                (targets, self.x_ptr[K], engine.F16, M, engine.F16, engine.F32,
-                 engine.FUSE_GATE_UP_SILU if silu and len(targets) == 2 else 0)
-                for targets, K in groups]))
+                    groups.append(([target], K, name))
+            items = []
+            for targets, K, name in groups:
+                fused = silu and len(targets) == 2
+                x = self.y_ptr["gate_proj"] if silu and name == "down_proj" and "gate_proj" in self.y_ptr else self.x_ptr[K]
+                items.append((targets, x, engine.F16, M, engine.F16, engine.F32, engine.FUSE_GATE_UP_SILU if fused else 0))
+            out.append(engine.make_calls(items))
         return out
 
     def digest(self):
@@ -274,6 +279,8 @@ def measure_layer(ctx, work, M, steps, warmup, preheat_ms, fuse=True, silu=False
     run_steps(steps)
     kernel_ms, launches = ctx.profile_end()
     per_launch = ctx.profile_durations()
+    if launches % steps == 0:  # calls that went out together as one kernel count as one launch
+        launches_per_step = int(launches) // steps
     for g in graphs or []:
         ctx.graph_destroy(g)
     # kernel time of each step (its launches, and the slice reductions some of them carry)
@@ -787,7 +794,11 @@ def main():
                         help="replay each step from a recorded HIP graph (one host call per step) in "
                              "the timed pass; the per-kernel pass stays eager")
     parser.add_argument("--fused-mlp", action="store_true",
-                        help="gate|up launch applies silu(gate)*up (one output instead of two)")
+                        help="gate|up launch applies silu(gate)*up (one output instead of two) and down_proj "
+                             "reads that output")
+    parser.add_argument("--chain", action="store_true",
+                        help="with --fused-mlp: context option chain = 1, the gate|up-SiLU launch and "
+                             "down_proj go out as one kernel (three launches a step)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline legs")
     parser.add_argument("--no-secondary", action="store_true",
                         help="default workload only: leave out the verify / prefill / W8A8 figures")
@@ -817,9 +828,13 @@ def main():
     copies = {"layer_m1": args.copies, "config1": max(args.copies, 600), "lm_head": 2}[args.workload]
     if args.workload == "lm_head" and args.steps == 400 and args.warmup == 40:
         args.steps, args.warmup = 60, 6
+    if args.chain:
+        args.fused_mlp = True
     headline = args.workload == "layer_m1" and M == 1 and not (args.unfused or args.graph or args.fused_mlp)
     with_secondary = headline and not args.no_secondary
     ctx = engine.Context(0)  # raises without a GPU
+    if args.chain:
+        ctx.set_option("chain", "1")
     info = ctx.info()
     work = LayerWorkload(engine, ctx, shapes, copies, meta_kind, max(M, 8) if with_secondary else M,
                          args.verbose)
@@ -859,6 +874,7 @@ def main():
             "linears_per_step": len(shapes),
             "launches_per_step": launches_per_step,
             "gate_up_silu_fused": bool(args.fused_mlp),
+            "mlp_as_one_launch": bool(args.chain),
             "steps_replayed_from_graph": bool(args.graph),
             "algorithmic_bytes_per_step": step_bytes,
             "weight_copies_rotated": copies,
