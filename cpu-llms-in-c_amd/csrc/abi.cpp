@@ -91,6 +91,10 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "half_tiles") == 0) {  // "1" / "0": the half-tile form of the streaming launch always / never
+        ctx->half_tiles = !set ? -1 : strcmp(value, "0") != 0 ? 1 : 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "batch_invariant") == 0) {
         ctx->batch_invariant = set && strcmp(value, "0") != 0;
         return MI355Q_OK;
@@ -194,6 +198,7 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     if (status == hipSuccess) status = hipHostMalloc((void **)&ctx->chain_gave_up, sizeof(uint32_t), hipHostMallocDefault);
     if (status == hipSuccess) *ctx->chain_gave_up = 0u;
     ctx->chain_spin_limit = kChainSpinLimitDefault;
+    ctx->half_tiles = -1;
     if (status == hipSuccess) status = q4_stream_scratch_init(ctx);  // this device is current
     uint32_t xcds = 0;
     if (status == hipSuccess) status = probe_columns_share_xcd(ctx, &ctx->columns_share_xcd, &xcds);

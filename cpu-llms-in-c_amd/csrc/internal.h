@@ -83,6 +83,7 @@ struct mi355q_context {
     // option "batch_invariant" = "1": streaming launches of up to eight activation rows take the
     // waves and K slices of the one-row launch, so that a row's result does not depend on the batch
     bool batch_invariant;
+    int half_tiles;  // option "half_tiles": -1 the launch decides, 1 wherever the kernel can, 0 never
     bool gemm_plain_loads;  // option "gemm_loads" = "plain": the 17-tile GEMM shape with compiler-managed weight loads
     int w8a8_tiles;       // option "w8a8" = "1" .. "4": tiles per W8A8 workgroup (0: chosen by the launch)
     bool lds_raised[16];  // q4_gemm_pipe_kernel instantiations whose dynamic LDS limit has been raised
@@ -203,6 +204,9 @@ struct Q4LinearArgs {
     // live in the library's fixed device array (q4_stream_scratch_init), sizes beyond it are
     // refused, and so is per-kernel profiling (which creates events).
     bool no_alloc;
+    // the launch shape in whole tiles only (the caller runs the streaming workgroup inside a kernel
+    // of its own that has no half-tile form)
+    bool whole_tiles;
     // Columns of an activation row when they are fewer than the weight's: K / 2 (a multiple of
     // 128, one target).  The weight's second half of columns then meets the same row again from
     // its start - how the doubled [high | low nibble] weight of an 8-bit matrix is applied.  0: K.

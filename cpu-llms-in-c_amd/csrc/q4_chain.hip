@@ -79,10 +79,12 @@ int q4_chain_linear(mi355q_context *ctx, const Q4LinearArgs &gate_up, const Q4Li
                     size_t error_capacity)
 {
     StreamPlan a, b;
+    Q4LinearArgs second = down;
+    second.whole_tiles = true;
     int status = q4_stream_plan(ctx, gate_up, a, error, error_capacity);
-    if (status == MI355Q_OK) status = q4_stream_plan(ctx, down, b, error, error_capacity);
+    if (status == MI355Q_OK) status = q4_stream_plan(ctx, second, b, error, error_capacity);
     if (status != MI355Q_OK) return status;
-    if (a.shape.mp != b.shape.mp || a.shape.tb != 2 || a.shape.waves != 4 || a.shape.depth != 2 || a.shape.slices != 1u ||
+    if (a.shape.half || b.shape.half || a.shape.mp != b.shape.mp || a.shape.tb != 2 || a.shape.waves != 4 || a.shape.depth != 2 || a.shape.slices != 1u ||
         b.shape.tb != (b.shape.mp <= 2 ? 1 : 2) || b.shape.waves != 4 || b.shape.depth != 2 ||
         (b.shape.slices > 1u && b.p.arrivals == nullptr)) {
         set_error(error, error_capacity, "q4 chained launch: launch shapes changed between the check and the plan");

@@ -81,6 +81,14 @@ __global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
     stream_workgroup<MP, TB, D, W, BF, WRAP, kStreamPlain>(p, ChainParams{}, blockIdx.x, blockIdx.y, lds);
 }
 
+// The half-tile form (see stream_workgroup): MP operand rows = two per activation row.
+template <int MP, int W, bool BF>
+__global__ void __launch_bounds__(64 * W) q4_stream_half_kernel(const StreamParams p)
+{
+    extern __shared__ uint4 lds[];
+    stream_workgroup<MP, 1, 2, W, BF, false, kStreamPlain, true>(p, ChainParams{}, blockIdx.x, 0u, lds);
+}
+
 // Adds the slices' partial sums in slice order (a fixed order) and applies the
 // epilogue.  One thread per output element of all targets.
 __global__ void __launch_bounds__(256) q4_stream_reduce_kernel(const StreamParams p)
@@ -202,6 +210,36 @@ static hipError_t launch_one(mi355q_context *ctx, const StreamParams &p)
     return launch(ctx, q4_stream_kernel<MP, TB, D, W, false>, grid, dim3(64u * W), lds, q);
 }
 
+template <int MP, int W>
+static hipError_t launch_half(mi355q_context *ctx, const StreamParams &p)
+{
+    uint32_t blocks = 0;
+    for (uint32_t t = 0; t < p.targets; ++t) blocks += 2u * p.NT[t];
+    StreamParams q = p;
+    q.columns = blocks;
+    const size_t lds = stream_lds_bytes(MP, 1, 2, W);
+    if (q.meta_bf16) return launch(ctx, q4_stream_half_kernel<MP, W, true>, dim3(blocks), dim3(64u * W), lds, q);
+    return launch(ctx, q4_stream_half_kernel<MP, W, false>, dim3(blocks), dim3(64u * W), lds, q);
+}
+
+// the half-tile kernels: operand rows 2, 4 or 8 (one, two or four activation rows), four or eight waves
+static hipError_t launch_half_shape(mi355q_context *ctx, const StreamParams &p, const StreamShape &shape, bool *missing)
+{
+    *missing = false;
+    switch (shape.mp * 100 + shape.waves) {
+    case 204: return launch_half<2, 4>(ctx, p);
+    case 208: return launch_half<2, 8>(ctx, p);
+    case 216: return launch_half<2, 16>(ctx, p);
+    case 404: return launch_half<4, 4>(ctx, p);
+    case 408: return launch_half<4, 8>(ctx, p);
+    case 804: return launch_half<8, 4>(ctx, p);
+    case 808: return launch_half<8, 8>(ctx, p);
+    default: break;
+    }
+    *missing = true;
+    return hipSuccess;
+}
+
 // *missing is set when no kernel is built for the shape (nothing is launched then)
 template <int MP>
 static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const StreamShape &shape, bool *missing)
@@ -255,6 +293,7 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         return shape;
     }
     shape.mp = mp;
+    shape.half = false;
     shape.tb = 1;
     shape.depth = 2;
     uint32_t slices = 1;
@@ -386,6 +425,28 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
     if (shape.tb > 1 && shape.waves > 8) shape.waves = 8;  // sixteen waves exist for single tiles only
     while (shape.waves > 2 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u)
         shape.waves /= 2;
+    // The half-tile form (stream_workgroup): for one 16-bit activation row against few tiles of
+    // middling rows - a launch that cannot fill the chip with whole tiles (the 27B o projection:
+    // 320 tiles of 48 steps on 256 compute units).  Twice the workgroups, four waves each.
+    // Measured per launch, whole tiles against half tiles (interleaved on one box): o at one row
+    // 6.7-7.1 us against 6.3 (four waves; eight 6.6, sixteen 8.6), at two rows 7.16 / 7.04; down
+    // (136 steps, otherwise three K slices) 13.2-13.4 / 13.0-13.9: no gain, it keeps its slices;
+    // q|k|v and gate|up lose (6.4 / 6.9-7.9, 18.7 / 19.9-24.6).
+    // Option "half_tiles": "1" wherever the kernel can (up to four rows), "0" never.
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    const bool half_possible = !pair && !subset && !a.fuse_silu && a.x_columns == 0 && rows <= 4u && first.T % 2u == 0u &&
+                               first.K % kStepColumns == 0u && !ctx->batch_invariant && !a.no_alloc && !a.whole_tiles;
+    const bool half_pays = rows == 1u && tiles <= cus + cus / 2u && first.T >= 32u && first.T < 96u && ctx->force_stream[0] <= 0;
+    if (half_possible && ctx->half_tiles != 0 && (ctx->half_tiles == 1 || half_pays)) {
+        shape.half = true;
+        shape.mp = 2;
+        while ((uint32_t)shape.mp < 2u * rows) shape.mp *= 2;
+        shape.tb = 1;
+        shape.depth = 2;
+        shape.waves = ctx->force_stream[0] > 0 ? ctx->force_stream[2] : 4;
+        shape.slices = 1;
+        shape.slice_steps = first.T / 2u;
+    }
     uint32_t block = 0;
     for (uint32_t t = 0; t < a.count; ++t) {
         const Q4Device &w = *a.targets[t].w;
@@ -397,7 +458,7 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
         p.NT[t] = subset ? (a.row_count + kTileRows - 1) / kTileRows : w.NT;
         p.stride[t] = w.NT;
         p.first_block[t] = block;
-        block += (p.NT[t] + shape.tb - 1) / shape.tb;
+        block += shape.half ? 2u * p.NT[t] : (p.NT[t] + shape.tb - 1) / shape.tb;
     }
     if (a.fuse_silu) p.first_block[1] = 0xffffffffu;  // every workgroup starts from target 0
     p.fuse_silu = a.fuse_silu;
@@ -406,9 +467,9 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
     p.targets = a.count;
     p.M = a.M;
     p.K = x_columns;
-    p.T = first.T;
+    p.T = shape.half ? first.T / 2u : first.T;  // half-tile form: pairs of steps
     p.wrap_steps = a.x_columns ? a.x_columns / kStepColumns : 0xffffffffu;
-    p.rows = rows;
+    p.rows = shape.half ? 2u * rows : rows;     // half-tile form: operand rows, two per activation row
     p.slice_steps = shape.slice_steps;
     p.slices = shape.slices;
     uint32_t counted_columns = 0;  // workgroup columns that count arrivals in this launch
@@ -451,7 +512,7 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
     p.residual_is_bias = a.residual_is_bias;
     p.meta_bf16 = first.meta_kind == MI355Q_META_BF16_PLANES;
 
-    const size_t lds = stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves);
+    const size_t lds = stream_lds_bytes(shape.mp, shape.tb, shape.depth, shape.waves);
     if (lds + 64u > 64u * 1024u) {  // a few bytes of static LDS besides
         set_error(error, error_capacity, "q4 stream kernel: %zu bytes of LDS needed (K=%u, rows=%u)",
                   lds, first.K, rows);
@@ -475,11 +536,14 @@ int q4_stream_linear(mi355q_context *ctx, const Q4LinearArgs &a, char *error, si
     const StreamShape &shape = plan.shape;
     if (ctx->trace)
         fprintf(stderr, "mi355q: q4 stream rows=%u tiles=%u steps=%u -> %d tiles x %d waves per workgroup, "
-                        "depth %d, %u slices of %u steps\n", plan.rows, plan.tiles, p.T, shape.tb,
+                        "depth %d, %u slices of %u steps%s\n", plan.rows, plan.tiles, p.T, shape.tb,
                 shape.waves, shape.depth, shape.slices,
-                shape.slice_steps);
+                shape.slice_steps, shape.half ? " (half tiles, pairs of steps)" : "");
     hipError_t launched;
     bool missing = false;
+    if (shape.half)
+        launched = launch_half_shape(ctx, p, shape, &missing);
+    else
     switch (shape.mp) {
     case 1: launched = launch_shape<1>(ctx, p, shape, &missing); break;
     case 2: launched = launch_shape<2>(ctx, p, shape, &missing); break;

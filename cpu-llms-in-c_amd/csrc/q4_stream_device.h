@@ -129,11 +129,24 @@ struct ChainParams {
 // it was; its sixteen-wave form fits two workgroups on a compute unit only below 65 registers)
 // ROLE: kStreamPlain, or one side of a chained pair of linears (see ChainParams).  block_x and
 // block_y are the workgroup's column and row among the workgroups of its linear.
-template <int MP, int TB, int D, int W, bool BF, bool WRAP, int ROLE>
+// HALF: a workgroup takes eight of a tile's sixteen rows and two 128-column steps at a time: the
+// lanes that would hold rows 8-15 of a step hold the workgroup's eight rows of the NEXT step
+// instead (a per-lane address offset of one step; the tile layout in memory is what it was), and
+// the activations of the two steps travel as two "rows" of the matrix instruction's first
+// operand, so that accumulator row 2m + h of a lane is (activation row m) x (the lane's step h).
+// A lane's own step is h = r / 8: lanes r < 8 keep the even accumulator rows, lanes r >= 8 the
+// odd ones, and output (m, n) is the sum of the two.  Twice the workgroups with half the steps
+// each and nothing to exchange between them: for matrices of few tiles and long rows (the 27B
+// o and down projections at one and two rows), whose launches are bound by the chain of memory
+// round trips of a wave and not by bandwidth.  MP counts the operand rows (2 per activation
+// row); p.T counts pairs of steps; p.rows = 2 M.  One tile, no K slices, no fused pair, no row
+// subset, 16-bit activations.
+template <int MP, int TB, int D, int W, bool BF, bool WRAP, int ROLE, bool HALF = false>
 __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const ChainParams &chain,
                                                  const uint32_t block_x, const uint32_t block_y, uint4 *const lds)
 {
     constexpr int NJ = MP < 4 ? MP : 4;
+    static_assert(!HALF || (TB == 1 && MP >= 2 && !WRAP && ROLE == kStreamPlain), "what the half-tile form covers");
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -164,7 +177,8 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const Ch
                  "s"(meta_target), "s"(meta_up));
     // tiles per target and workgroup: TB, or TB/2 of each of the two fused targets
     const uint32_t span_tiles = fuse_silu ? (TB > 1 ? TB / 2u : 1u) : TB;
-    const uint32_t tile0 = (block_x - first_block) * span_tiles;
+    const uint32_t tile0 = HALF ? (block_x - first_block) / 2u : (block_x - first_block) * span_tiles;
+    const uint32_t row_half = HALF ? (block_x - first_block) & 1u : 0u;  // HALF: rows 8 * row_half .. + 7 of the tile
 
     // LDS: every wave owns R slots of activations, one per step it has in flight (a step's
     // activations are read by the one wave that takes the step: nothing is shared, so there is
@@ -209,10 +223,19 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const Ch
             meta_lane[tb] = ((row / kTileRows) * 16u + row % kTileRows) * (uint32_t)sizeof(uint2);
             continue;
         }
+        if constexpr (HALF) {
+            // lane (r, kq): row 8 * row_half + r % 8 of the tile, in step 2 * pair + r / 8
+            const uint32_t row = 8u * row_half + (r & 7u), later = r >> 3;
+            codes_lane[tb] = (tile * 64u + kq * 16u + row) * (uint32_t)sizeof(uint4) + later * stride * 64u * (uint32_t)sizeof(uint4);
+            meta_lane[tb] = (tile * 16u + row) * (uint32_t)sizeof(uint2) + later * stride * 16u * (uint32_t)sizeof(uint2);
+            continue;
+        }
         codes_lane[tb] = (tile * 64u + lane) * (uint32_t)sizeof(uint4);
         meta_lane[tb] = (tile * 16u + r) * (uint32_t)sizeof(uint2);
     }
-    const size_t codes_step = (size_t)stride * 64u * sizeof(uint4), meta_step = (size_t)stride * 16u * sizeof(uint2);
+    // bytes from one of the wave's steps (HALF: pairs of steps) to the next in memory
+    const size_t codes_step = (size_t)stride * 64u * sizeof(uint4) * (HALF ? 2u : 1u),
+                 meta_step = (size_t)stride * 16u * sizeof(uint2) * (HALF ? 2u : 1u);
 
     // where lane l reads the activations it brings into a slot: entry e = l + 64 b of the slot
     // is (octet e / MP, row e % MP).  Rows beyond the last repeat it and octets beyond the
@@ -224,7 +247,10 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const Ch
         uint32_t o = e / MP, mrow = e % MP;
         o = o < 16u ? o : 15u;
         mrow = mrow < rows ? mrow : rows - 1u;
-        x_lane[b] = (mrow * K + o * 8u) * (uint32_t)sizeof(_Float16);
+        if constexpr (HALF)  // operand row 2 m + h: activation row m, the pair's step h
+            x_lane[b] = ((mrow >> 1) * K + (mrow & 1u) * kStepColumns + o * 8u) * (uint32_t)sizeof(_Float16);
+        else
+            x_lane[b] = (mrow * K + o * 8u) * (uint32_t)sizeof(_Float16);
         // K is a multiple of 64: when it is an odd one, the upper half of the last step does not
         // exist (its codes and metadata are zero); the lane reads the lower half again
         x_lane_tail[b] = x_lane[b] - (o >= 8u ? 64u * (uint32_t)sizeof(_Float16) : 0u);
@@ -271,7 +297,7 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const Ch
         auto fetch = [&](uint32_t step, auto slot_c, StepData<TB> &slot) {
             constexpr uint32_t slot_bytes = decltype(slot_c)::value * SLAB * (uint32_t)sizeof(uint4);
             const uint32_t x_step = WRAP && step >= wrap_steps ? step - wrap_steps : step;
-            uint64_t x_at = (uint64_t)((const char *)x + (size_t)x_step * (kStepColumns * sizeof(_Float16)));
+            uint64_t x_at = (uint64_t)((const char *)x + (size_t)x_step * ((HALF ? 2u : 1u) * kStepColumns * sizeof(_Float16)));
             asm volatile("" : "+s"(x_at));
             const bool tail_step = odd_tail && step + 1u == T;
             if constexpr (ROLE == kChainConsumer) fetch_weights(step, slot);
@@ -500,6 +526,32 @@ __device__ __forceinline__ void stream_workgroup(const StreamParams &p, const Ch
 #pragma unroll
         for (int j = 0; j < NJ; ++j) red[((wave * TB + tb) * NJ + j) * 64u + lane] = acc[tb][j];
     __syncthreads();
+    if constexpr (HALF) {
+        // lane l = (r < 8, kq): outputs n = 16 tile + 8 row_half + r of the activation rows
+        // m = 2 kq + j / 2 (j even): the waves' sums of operand row 2m at lane l (step h = 0) and
+        // of operand row 2m + 1 at lane l + 8 (h = 1), each added in wave order, then the two
+        const uint32_t l = threadIdx.x & 63u;
+        if (threadIdx.x >= 64u || (l & 8u) != 0u || tile0 >= NT) return;
+        const uint32_t n = tile0 * kTileRows + 8u * row_half + (l & 7u);
+        if (n >= N) return;
+#pragma unroll
+        for (int j = 0; j < NJ; j += 2) {
+            const uint32_t m = 2u * (l >> 4) + (uint32_t)j / 2u;
+            if (2u * m >= p.rows) continue;
+            float even = 0.0f, odd = 0.0f;
+#pragma unroll
+            for (int w = 0; w < W; ++w) even += red[((w * TB) * NJ + j) * 64u + l];
+#pragma unroll
+            for (int w = 0; w < W; ++w) odd += red[((w * TB) * NJ + j + 1) * 64u + l + 8u];
+            float value = even + odd;
+            const size_t at = (size_t)m * N + n;
+            if (p.row_scale) value *= p.row_scale[m];
+            if (p.residual[target])
+                value += load_as_float(p.residual[target], p.residual_dtype, p.residual_is_bias ? n : at);
+            store_from_float(p.y[target], p.y_dtype, at, value);
+        }
+        return;
+    }
     for (uint32_t e = threadIdx.x; e < TB * 64u; e += 64u * W) {
         const uint32_t tb = e >> 6, l = e & 63u;
         const uint32_t slot_target = p.fuse_silu ? tb / span_tiles : target;

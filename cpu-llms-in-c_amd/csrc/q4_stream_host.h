@@ -10,6 +10,9 @@ namespace mi355q {
 struct StreamShape {
     int mp, tb, depth, waves;
     uint32_t slices, slice_steps;
+    // the half-tile form: twice the workgroups, eight rows and two steps at a time each; mp then
+    // counts the matrix instruction's operand rows (two per activation row)
+    bool half;
 };
 
 // What one streaming launch needs: the kernel's parameters and its launch shape.

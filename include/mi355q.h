@@ -133,6 +133,10 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *                                               142-248; tests/qwen38_m3_prefill_parity_test.c:115-199):
  *                                               the launch takes the waves and K slices of the one-row
  *                                               launch instead of the fastest ones for its row count
+ *   "half_tiles" = "1" / "0"                    the streaming launch's half-tile form (a workgroup takes
+ *                                               eight of a tile's rows and two 128-column steps at a
+ *                                               time) wherever the kernel has it (up to four 16-bit
+ *                                               rows) / never; unset: where it measured faster
  *   "chain" = "1"                               mi355q_q4_linear_sequence runs gate|up-SiLU and the
  *                                               linear that reads its output as ONE launch (see there;
  *                                               also MI355Q_CHAIN=1 in the environment).  Off by default:

@@ -4,7 +4,8 @@ waits, 128 columns at a time, for the first half's outputs (the reference encode
 kernels into one command buffer, qwen38_m3_layer.m:314-336; qwen38_q4.metal:129-191).
 
 The one-launch form is behind the context option "chain" = "1".  Gates: the one-launch pair is
-bit-equal to the same two calls as two launches, and both match the oracle: h = silu(gate . x) * (up . x) rounded to fp16, and
+bit-equal to the same two calls as two launches of whole tiles (the launch shapes the pair shares;
+option "half_tiles" = "0" keeps the two-launch form on them), and both match the oracle: h = silu(gate . x) * (up . x) rounded to fp16, and
 y = down . h (+ residual) on the GPU's own h, within the Q4 gate of 1e-3."""
 import numpy as np
 import pytest
@@ -84,6 +85,7 @@ def test_27b_mlp_one_launch_equals_two(engine, oracle, gpu, force, mlp_27b, M):
     the two launches, both right."""
     print(f"chained 27B MLP M={M}", flush=True)
     before = gpu.get("chained_launches")
+    force("half_tiles", "0")
     h0, y0 = mlp_27b.run(M, residual=True)
     assert gpu.get("chained_launches") == before  # off unless asked for
     force("chain", "1")

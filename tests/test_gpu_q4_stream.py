@@ -514,3 +514,61 @@ def test_recorded_sequence_replays(engine, oracle, gpu):
         for w in weights:
             w.destroy()
         gpu.close()
+
+
+HALF_CASES = [
+    # name, [N per target], K, M, x dtype, residual
+    ("o_m1", [5120], 6144, 1, "F16", False),
+    ("o_m2_residual", [5120], 6144, 2, "F16", True),
+    ("down_m1", [5120], 17408, 1, "F16", False),
+    ("down_m2_bf16", [5120], 17408, 2, "BF16", True),
+    ("ragged_m1", [1000], 1536, 1, "F16", False),
+    ("ragged_m3", [1000], 1536, 3, "F16", True),
+    ("m4", [528], 2048, 4, "BF16", False),
+    ("three_targets_m2", [640, 328, 16], 1024, 2, "F16", True),
+]
+
+
+@pytest.mark.parametrize("name,rows,K,M,x_dtype,with_residual", HALF_CASES, ids=[c[0] for c in HALF_CASES])
+def test_half_tile_form(engine, oracle, gpu, force, name, rows, K, M, x_dtype, with_residual):
+    """The half-tile form of the streaming launch (eight rows of a tile and two 128-column steps at
+    a time per workgroup; what o_proj and down_proj of the 27B layer take at one and two rows):
+    forced on for every shape here, against the oracle and against the whole-tile launch of the
+    same call (which adds the same products in another order: equal within the gate, and a
+    second launch of the half-tile form repeats its own bits)."""
+    x_dtype = getattr(engine, x_dtype)
+    kind = engine.META_BF16_PLANES
+    images = [engine.synth_q4_affine(400 + i, 0.02, N, K, kind) for i, N in enumerate(rows)]
+    weights = [gpu.q4_prepare(*image, N, K, kind) for image, N in zip(images, rows)]
+    x = make_x(engine, 410, M, K, x_dtype)
+    residuals = [engine.synth_normal_f32(420 + i, 1.0, M * N).reshape(M, N) if with_residual else None
+                 for i, N in enumerate(rows)]
+    pointers = []
+    try:
+        print(f"half tile case {name}", flush=True)
+        x_ptr = gpu.to_device(x)
+        y_ptrs = [gpu.alloc(M * N * 4) for N in rows]
+        r_ptrs = [gpu.to_device(r) if r is not None else None for r in residuals]
+        pointers = [x_ptr] + y_ptrs + [p for p in r_ptrs if p]
+        calls = engine.make_calls([([(w, y, r) for w, y, r in zip(weights, y_ptrs, r_ptrs)], x_ptr, x_dtype, M,
+                                    engine.F32, engine.F32)])
+        results = {}
+        for mode in ("0", "1", "1 again"):
+            force("half_tiles", mode[0])
+            for y_ptr, N in zip(y_ptrs, rows):
+                gpu.upload(y_ptr, np.full((M, N), np.nan, dtype=np.float32))
+            gpu.q4_sequence(calls)
+            gpu.sync()
+            results[mode] = [gpu.download(y_ptr, (M, N), np.float32) for y_ptr, N in zip(y_ptrs, rows)]
+    finally:
+        for pointer in pointers:
+            gpu.free(pointer)
+        for weight in weights:
+            weight.destroy()
+    for i, N in enumerate(rows):
+        reference = oracle.q4_linear(*images[i], kind, N, K, x, x_dtype, M)
+        if with_residual:
+            reference = reference + residuals[i]
+        assert q4_relative_error(results["1"][i], reference) <= TOLERANCE
+        assert q4_relative_error(results["0"][i], reference) <= TOLERANCE
+        assert np.array_equal(results["1"][i].view(np.uint32), results["1 again"][i].view(np.uint32))
