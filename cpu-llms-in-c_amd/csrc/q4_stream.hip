@@ -435,7 +435,7 @@ int q4_stream_plan(mi355q_context *ctx, const Q4LinearArgs &a, StreamPlan &plan,
     // Option "half_tiles": "1" wherever the kernel can (up to four rows), "0" never.
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     const bool half_possible = !pair && !subset && !a.fuse_silu && a.x_columns == 0 && rows <= 4u && first.T % 2u == 0u &&
-                               first.K % kStepColumns == 0u && !ctx->batch_invariant && !a.no_alloc && !a.whole_tiles;
+                               first.K % kStepColumns == 0u && !ctx->batch_invariant && !a.whole_tiles;
     const bool half_pays = rows == 1u && tiles <= cus + cus / 2u && first.T >= 32u && first.T < 96u && ctx->force_stream[0] <= 0;
     if (half_possible && ctx->half_tiles != 0 && (ctx->half_tiles == 1 || half_pays)) {
         shape.half = true;

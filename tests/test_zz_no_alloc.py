@@ -27,6 +27,7 @@ CASES = [
     ("down_sliced_f32_residual", 5120, 17408, "F32", True, (4, 2)),
     ("few_tiles_long_rows", 528, 17472, "F32", False, (6, 1)),
     ("gate_unsliced", 17408, 5120, "F16", False, (2, 1)),
+    ("o_half_tiles_at_one_row", 5120, 6144, "F16", True, (2, 1)),
     ("ragged_small", 100, 192, "F32", True, (8, 3)),
 ]
 
