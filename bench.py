@@ -524,10 +524,11 @@ Q8_AFFINE = {"N": 25600, "K": 5120}  # gate/up projection of the H3 text conditi
 
 def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
     """Affine-Q8 g64 linear (minimax_h3_q8_gemm_bf16_meta's format) of the conditioner's gate shape:
-    GB/s of the weight image at M = 1, TFLOP/s at prefill M.  The weight is one Q4 weight of twice
-    the columns here (high nibbles | low nibbles) whose second half meets the activation row again
-    from its start, so a linear is one Q4 linear.  Random codes and metadata: timing only,
-    parity is the GPU tests' business."""
+    GB/s of the weight image at M = 1, TFLOP/s at prefill M.  Up to 16 rows the weight is one Q4
+    weight of twice the columns (high nibbles | low nibbles) whose second half meets the activation
+    row again from its start, so a linear is one Q4 streaming linear; above, the pipelined GEMM
+    kernel multiplies the bytes themselves (a second copy of the weight, in GEMM tiles).  Random
+    codes and metadata: timing only, parity is the GPU tests' business."""
     N, K = Q8_AFFINE["N"], Q8_AFFINE["K"]
     rng = np.random.default_rng(77)
     quants = rng.integers(0, 256, size=N * K, dtype=np.uint8)
@@ -565,8 +566,8 @@ def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
             entry.update({"tflops": round(achieved, 1),
                           "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": F16_MFMA_PEAK_TFLOPS,
                                        "unit": "TFLOP/s", "frac": round(achieved / F16_MFMA_PEAK_TFLOPS, 4),
-                                       "kernel": "q4_gemm_pipe_kernel over [high | low nibbles] x [x | x]: the matrix "
-                                                 "units do 2x the algorithmic flops counted here"}})
+                                       "kernel": "q4_gemm_pipe_kernel<128, 4, false, false, true>: 8-bit codes, "
+                                                 "16 tiles per workgroup"}})
         out["q8_affine_g64_m%d" % M] = entry
         ctx.free(x_ptr)
         ctx.free(y_ptr)

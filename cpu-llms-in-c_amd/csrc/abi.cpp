@@ -91,6 +91,11 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "q8_gemm") == 0) {  // "doubled": no 8-bit GEMM kernel; "native" or unset: use it where it applies
+        if (set && strcmp(value, "doubled") != 0 && strcmp(value, "native") != 0) return MI355Q_ERROR_INVALID;
+        ctx->q8_gemm_doubled = set && strcmp(value, "doubled") == 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "half_tiles") == 0) {  // "1" / "0": the half-tile form of the streaming launch always / never
         ctx->half_tiles = !set ? -1 : strcmp(value, "0") != 0 ? 1 : 0;
         return MI355Q_OK;

@@ -42,6 +42,12 @@ struct Q4Device {
     uint32_t N, K;  // logical shape
     uint32_t NT, T; // tiles of 16 rows, steps of 128 columns
     int meta_kind;
+    // Only when this is the doubled form [high nibbles | low nibbles] of an 8-bit weight whose
+    // columns are whole 128-column steps: the bytes themselves in tiles of the same rows and
+    // columns, [T/2][NT][2][64] of 16 bytes, and their fp16 {scale, bias} records [T/2][NT][16],
+    // for the GEMM kernel that multiplies 8-bit codes directly.  Owned by the 8-bit weight.
+    uint4 *codes8;
+    uint2 *meta8;
 };
 
 }  // namespace mi355q
@@ -84,6 +90,7 @@ struct mi355q_context {
     // waves and K slices of the one-row launch, so that a row's result does not depend on the batch
     bool batch_invariant;
     int half_tiles;  // option "half_tiles": -1 the launch decides, 1 wherever the kernel can, 0 never
+    bool q8_gemm_doubled;   // option "q8_gemm" = "doubled": 8-bit weights take the Q4 GEMM kernels on their doubled form
     bool gemm_plain_loads;  // option "gemm_loads" = "plain": the 17-tile GEMM shape with compiler-managed weight loads
     int w8a8_tiles;       // option "w8a8" = "1" .. "4": tiles per W8A8 workgroup (0: chosen by the launch)
     bool lds_raised[16];  // q4_gemm_pipe_kernel instantiations whose dynamic LDS limit has been raised

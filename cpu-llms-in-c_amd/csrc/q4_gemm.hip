@@ -40,6 +40,7 @@ extern template __global__ void q4_gemm_pipe_kernel<128, 4, false, false>(const 
 extern template __global__ void q4_gemm_pipe_kernel<128, 4, true, false>(const GemmParams);
 extern template __global__ void q4_gemm_pipe_kernel<128, 4, true, true>(const GemmParams);
 extern template __global__ void q4_gemm_pipe_kernel<128, 5, false, false>(const GemmParams);
+extern template __global__ void q4_gemm_pipe_kernel<128, 4, false, false, true>(const GemmParams);  // 8-bit codes
 
 // Adds the K splits in split order (a fixed order) and applies the epilogue.  WIDE: a thread
 // takes four adjacent outputs of one row (N a multiple of 4, y 16-byte aligned): 16-byte loads
@@ -127,6 +128,20 @@ static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &
     return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT>, grid, dim3(256), bytes, p);
 }
 
+// The 16-tile shape on 8-bit codes.
+static hipError_t launch_pipe_bytes(mi355q_context *ctx, dim3 grid, const GemmParams &p)
+{
+    constexpr size_t bytes = pipe_lds_bytes(128);
+    constexpr int slot = 14;
+    if (!ctx->lds_raised[slot]) {
+        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, 4, false, false, true>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (status != hipSuccess) return status;
+        ctx->lds_raised[slot] = true;
+    }
+    return launch(ctx, q4_gemm_pipe_kernel<128, 4, false, false, true>, grid, dim3(256), bytes, p);
+}
+
 // The 17-tile shape with compiler-managed weight loads (option "gemm_loads" = "plain").
 static hipError_t launch_pipe_plain(mi355q_context *ctx, dim3 grid, const GemmParams &p)
 {
@@ -174,14 +189,24 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         p.x = fp16_rows;
         row_scale = scales;
     }
+    // The doubled form of an 8-bit weight whose activation row the kernels would read twice: the
+    // kernel for 8-bit codes reads the bytes themselves instead, one pass over the row, half the
+    // matrix instructions.  It is the pipelined kernel, with that kernel's conditions.
+    const bool bytes_native = w.codes8 != nullptr && a.x_columns != 0 && !ctx->q8_gemm_doubled &&
+                              (uint64_t)rows * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
+    const uint32_t T = bytes_native ? w.T / 2u : w.T;
+    if (bytes_native) {
+        p.codes = w.codes8;
+        p.meta = w.meta8;
+    }
     p.y = converted_x ? ctx->stage[6] : a.targets[target].y;
     p.residual = converted_x ? nullptr : a.targets[target].residual;
     p.M = rows;
     p.N = w.N;
     p.K = x_columns;
-    p.wrap_steps = a.x_columns ? a.x_columns / kStepColumns : 0xffffffffu;
+    p.wrap_steps = a.x_columns && !bytes_native ? a.x_columns / kStepColumns : 0xffffffffu;
     p.NT = w.NT;
-    p.T = w.T;
+    p.T = T;
     p.y_dtype = converted_x ? MI355Q_F32 : a.y_dtype;
     p.residual_dtype = a.residual_dtype;
     p.residual_is_bias = a.residual_is_bias;
@@ -205,7 +230,9 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     static const Variant variants[] = {
         {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
         {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
-        {128, 4, 0, 1, 0.0, 0.0, 1.493}, {128, 4, 1, 1, 0.0, 0.0, 1.675}, {128, 5, 0, 1, 0.0, 0.0, 1.849}};
+        {128, 4, 0, 1, 0.0, 0.0, 1.493}, {128, 4, 1, 1, 0.0, 0.0, 1.675}, {128, 5, 0, 1, 0.0, 0.0, 1.849},
+        {128, 4, 0, 1, 0.0, 0.0, 1.60}};  // 9: the 16-tile shape on 8-bit codes, and only for them
+    constexpr int kBytesVariant = 9;
     // A round of the pipelined kernel that fills only the fraction r of the compute units runs
     // faster than a full one: the chip is power limited, and up to about half of it the clock
     // stays near its maximum, from there it falls to the sustained clock of a full chip
@@ -223,14 +250,15 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)rows * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
         if (v >= 6 && !pipe_ok) continue;
+        if ((v == kBytesVariant) != bytes_native) continue;
         const Variant &c = variants[v];
         const uint32_t tpb = 4u * c.ntw + c.extra;
         const uint32_t slots = cus * (uint32_t)c.resident;
         const uint32_t m_blocks = (rows + c.bm - 1) / c.bm;
         const uint32_t n_blocks = (w.NT + tpb - 1) / tpb;
-        for (uint32_t want = 1; want <= 8u && want * 8u <= w.T + 7u; ++want) {
-            const uint32_t steps = (w.T + want - 1) / want;
-            const uint32_t splits = (w.T + steps - 1) / steps;
+        for (uint32_t want = 1; want <= 8u && want * 8u <= T + 7u; ++want) {
+            const uint32_t steps = (T + want - 1) / want;
+            const uint32_t splits = (T + steps - 1) / steps;
             const uint64_t groups = (uint64_t)n_blocks * m_blocks * splits;
             // one workgroup at peak: 64 matrix-instruction cycles per (tile, 16-row
             // fragment, step) and wave, at 2.4 GHz
@@ -266,21 +294,21 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     }
     // option "q4_gemm" = "VARIANT,SPLITS" for experiments
     if (ctx->force_gemm[1] >= 1 && ctx->force_gemm[0] < (int)(sizeof variants / sizeof variants[0]) &&
-        (ctx->force_gemm[0] < 6 || pipe_ok)) {
+        (ctx->force_gemm[0] < 6 || pipe_ok) && (ctx->force_gemm[0] == kBytesVariant) == bytes_native) {
         best = ctx->force_gemm[0];
         best_splits = (uint32_t)ctx->force_gemm[1];
     }
     if (ctx->trace)
-        fprintf(stderr, "mi355q: q4 gemm M=%u N=%u K=%u -> variant %d (BM=%d, %d tiles/wave%s), K split %u\n",
+        fprintf(stderr, "mi355q: q4 gemm M=%u N=%u K=%u -> variant %d (BM=%d, %d tiles/wave%s%s), K split %u\n",
                 rows, w.N, w.K, best, variants[best].bm, variants[best].ntw,
-                variants[best].extra ? " +1" : "", best_splits);
+                variants[best].extra ? " +1" : "", bytes_native ? ", 8-bit codes" : "", best_splits);
     const Variant &chosen = variants[best];
     const uint32_t tpb = 4u * chosen.ntw + chosen.extra;
     p.tiles_per_block = tpb;
     const uint32_t n_blocks = (w.NT + tpb - 1) / tpb;
     const uint32_t m_blocks = (rows + chosen.bm - 1) / chosen.bm;
-    p.steps_per_split = (w.T + best_splits - 1) / best_splits;
-    p.splits = (w.T + p.steps_per_split - 1) / p.steps_per_split;
+    p.steps_per_split = (T + best_splits - 1) / best_splits;
+    p.splits = (T + p.steps_per_split - 1) / p.steps_per_split;
     if (p.splits > 1u) {
         const size_t bytes = (size_t)p.splits * rows * w.N * sizeof(float);
         int status = ensure_stage(ctx, 4, bytes, error, error_capacity);
@@ -298,7 +326,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     case 5: launched = launch(ctx, q4_gemm_kernel<64, 2, true>, grid, dim3(256), 0, p); break;
     case 6: launched = launch_pipe<4, false>(ctx, grid, p); break;
     case 7: launched = ctx->gemm_plain_loads ? launch_pipe_plain(ctx, grid, p) : launch_pipe<4, true>(ctx, grid, p); break;
-    default: launched = launch_pipe<5, false>(ctx, grid, p); break;
+    case 8: launched = launch_pipe<5, false>(ctx, grid, p); break;
+    default: launched = launch_pipe_bytes(ctx, grid, p); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);

@@ -328,13 +328,23 @@ __global__ void __launch_bounds__(256, 2) q4_gemm_kernel(const GemmParams p)
 // are asm statements: asm keeps its source order, which is what places each in its slot between
 // the matrix instructions; the caller keeps dependent stages at least one instruction apart,
 // which covers the wait state a packed-fp16 result needs before a vector instruction reads it.
-template <int STAGE, int PIECE, int D, int NTX, class Codes, class Meta>
-__device__ __forceinline__ void dequant_stage(const Codes (&codes)[NTX], const Meta (&meta)[NTX],
+template <int STAGE, int PIECE, int D, bool Q8, int NC, int NTX, class Codes, class Meta>
+__device__ __forceinline__ void dequant_stage(const Codes (&codes)[NC], const Meta (&meta)[NTX],
                                               const NibbleMasks &masks, uint32_t (&merged)[4 * NTX],
                                               half2v (&centred)[4 * NTX], half2v (&out)[NTX][4])
 {
     constexpr int t = PIECE / 4, j = PIECE % 4;
-    if constexpr (STAGE == 0) {
+    if constexpr (STAGE == 0 && Q8) {
+        // 8-bit codes: a tile's step is two registers of sixteen bytes, quarter D the eight bytes
+        // D % 2 of register D / 2, a lane's eight weights in column order.  One byte permute
+        // builds fp16 1024 + code twice: bytes 2*(j%2) and 2*(j%2)+1 of the word under 0x64 each
+        // (`masks` holds the two selectors)
+        const Codes &both = codes[2 * t + D / 2];
+        const uint32_t word = D % 2 == 0 ? (j < 2 ? both.x : both.y) : (j < 2 ? both.z : both.w);
+        asm volatile("v_perm_b32 %0, %1, %2, %3"
+                     : "=v"(merged[PIECE])
+                     : "v"(word), "s"(0x64006400u), "v"((j & 1) ? masks.hi : masks.lo));
+    } else if constexpr (STAGE == 0) {
         uint32_t word = D == 0 ? codes[t].x : D == 1 ? codes[t].y : D == 2 ? codes[t].z : codes[t].w;
         if (j >= 2) word >>= 8;
         // fp16 1024 (64) twice, the code in the low (second) mantissa nibble
@@ -345,13 +355,22 @@ __device__ __forceinline__ void dequant_stage(const Codes (&codes)[NTX], const M
         // fp16 -1024 (-64) twice
         asm volatile("v_pk_add_f16 %0, %1, %2"
                      : "=v"(centred[PIECE])
-                     : "v"(merged[PIECE]), "s"((j & 1) ? 0xd400d400u : 0xe400e400u));
+                     : "v"(merged[PIECE]), "s"(((j & 1) && !Q8) ? 0xd400d400u : 0xe400e400u));
     } else {
         // scale = low half of the metadata word for both results, bias = high half for both
         asm volatile("v_pk_fma_f16 %0, %1, %2, %2 op_sel:[0,0,1] op_sel_hi:[1,0,1]"
                      : "=v"(out[t][j])
                      : "v"(centred[PIECE]), "v"(D < 2 ? meta[t].x : meta[t].y));
     }
+}
+
+// The selectors of the byte permute above, in vector registers: result bytes (code, 0x64, next
+// code, 0x64) from the word (bytes 4..7 of the permute's source pair) and the constant (0..3).
+__device__ __forceinline__ NibbleMasks byte_selectors()
+{
+    NibbleMasks m = {0x01050104u, 0x01070106u};
+    asm volatile("" : "+v"(m.lo), "+v"(m.hi));
+    return m;
 }
 
 // Where the pipelined kernel puts the dequantization of one quarter among the SLOTS matrix
@@ -446,9 +465,13 @@ __device__ __forceinline__ void load_to_lds(uint32_t lane_offset, const char *ba
                  : "memory", "m0");
 #pragma clang diagnostic pop
 }
+template <int IMMEDIATE = 0>
 __device__ __forceinline__ void load_x4(u32x4 &to, uint32_t lane_offset, const char *base)
 {
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(to) : "v"(lane_offset), "s"(base) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3"
+                 : "=v"(to)
+                 : "v"(lane_offset), "s"(base), "n"(IMMEDIATE)
+                 : "memory");
 }
 __device__ __forceinline__ void load_x2(u32x2 &to, uint32_t lane_offset, const char *base)
 {
@@ -459,7 +482,11 @@ __device__ __forceinline__ void load_x2(u32x2 &to, uint32_t lane_offset, const c
 // of asm statements under the kernel's own counted waits.  Slower, and the reference point for
 // the hand-scheduled form: both must give the same bits (a test compares them), which would
 // show a wait that no longer covers its loads after a change of compiler or of the schedule.
-template <int BM, int NTW, bool XT, bool PLAIN = false>
+// Q8: the weights are 8-bit codes in tiles of the same rows and columns (2 KiB per tile and step:
+// [step][tile][half][lane] of 16 bytes, half h = quarters 2h and 2h + 1, a lane's eight columns
+// of a quarter in order), with the same fp16 {scale, bias} records: one code register more per
+// tile and step, the same three vector instructions per pair of weights.
+template <int BM, int NTW, bool XT, bool PLAIN = false, bool Q8 = false>
 __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p)
 {
     extern __shared__ uint4 a_lds_raw[];  // [buffer][row][slot], slot = octet ^ (row % 16)
@@ -470,7 +497,10 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     constexpr int TPB = 4 * NTW + (XT ? 1 : 0);
     constexpr int NTX = NTW + (XT ? 1 : 0);
     constexpr int XI = MI / 4;  // row fragments of the shared tile per wave
-    constexpr int GROUP = AJ + 2 * NTX;  // loads one step's fetch puts in flight
+    constexpr int CW = Q8 ? 2 : 1;       // 16-byte code registers per tile and step
+    constexpr int NC = CW * NTX;
+    constexpr int PER = CW + 1;          // loads per tile and step: codes, then metadata
+    constexpr int GROUP = AJ + PER * NTX;  // loads one step's fetch puts in flight
     static_assert(2 * GROUP < 64, "the load counter holds 63");
     typedef __attribute__((address_space(3))) void *lds_ptr;
 
@@ -510,17 +540,17 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     for (int t = 0; t < NTX; ++t) {
         uint32_t tile = XT && t == NTX - 1 ? shared_tile : tile0 + t;
         tile = tile < p.NT ? tile : p.NT - 1u;
-        codes_offset[t] = (tile * 64u + lane) * (uint32_t)sizeof(uint4);
+        codes_offset[t] = (tile * (64u * CW) + lane) * (uint32_t)sizeof(uint4);
         meta_offset[t] = (tile * 16u + r) * (uint32_t)sizeof(uint2);
     }
     const uint32_t last_step = step_end - 1u;
     // the fetch pointers: they stop at the last step (later fetches repeat it: no branches)
     const char *x_next =
         (const char *)(p.x + (size_t)(step_begin >= p.wrap_steps ? step_begin - p.wrap_steps : step_begin) * kStepColumns) - 4096;
-    const char *codes_next = (const char *)(p.codes + (size_t)step_begin * p.NT * 64u);
+    const char *codes_next = (const char *)(p.codes + (size_t)step_begin * p.NT * (64u * CW));
     const char *meta_next = (const char *)(p.meta + (size_t)step_begin * p.NT * 16u);
     uint32_t fetch_step = step_begin;
-    const uint32_t codes_stride = p.NT * 64u * (uint32_t)sizeof(uint4);
+    const uint32_t codes_stride = p.NT * (64u * CW) * (uint32_t)sizeof(uint4);
     const uint32_t meta_stride = p.NT * 16u * (uint32_t)sizeof(uint2);
     const uint32_t lds_wave = (uint32_t)(uintptr_t)(lds_ptr)&a_lds(0)[(BM / 4) * wave][0] + 4096u;
     // Every global load of the loop is an asm statement, so the compiler inserts no waits of
@@ -530,20 +560,21 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     // before the wait that covers it (`landed` below marks that point for the compiler).
     // load number `load` of a step's fetch: the AJ pieces of the activation stage, then codes and
     // metadata of each tile
-    auto fetch_one = [&](auto load_c, uint32_t buffer, u32x4 (&codes)[NTX], u32x2 (&meta)[NTX]) {
+    auto fetch_one = [&](auto load_c, uint32_t buffer, u32x4 (&codes)[NC], u32x2 (&meta)[NTX]) {
         constexpr int load = decltype(load_c)::value;
+        constexpr int t = (load - AJ) / PER, part = (load - AJ) % PER;  // of a weight load
         if constexpr (load < AJ) {
             const uint32_t lds_base = lds_wave + buffer * (uint32_t)(BM * 16u * sizeof(uint4));
             load_to_lds<(load - AJ / 2) * 1024>(a_offset[load], x_next, lds_base);
         } else if constexpr (PLAIN) {
-            if constexpr ((load - AJ) % 2 == 0)
-                codes[(load - AJ) / 2] = *(const u32x4 *)(codes_next + codes_offset[(load - AJ) / 2]);
+            if constexpr (part < CW)
+                codes[CW * t + part] = *(const u32x4 *)(codes_next + codes_offset[t] + part * 1024);
             else
-                meta[(load - AJ) / 2] = *(const u32x2 *)(meta_next + meta_offset[(load - AJ) / 2]);
-        } else if constexpr ((load - AJ) % 2 == 0) {
-            load_x4(codes[(load - AJ) / 2], codes_offset[(load - AJ) / 2], codes_next);
+                meta[t] = *(const u32x2 *)(meta_next + meta_offset[t]);
+        } else if constexpr (part < CW) {
+            load_x4<part * 1024>(codes[CW * t + part], codes_offset[t], codes_next);
         } else {
-            load_x2(meta[(load - AJ) / 2], meta_offset[(load - AJ) / 2], meta_next);
+            load_x2(meta[t], meta_offset[t], meta_next);
         }
     };
     auto advance = [&]() {  // the pointers move on to the next step's fetch
@@ -556,11 +587,16 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         meta_next += more ? meta_stride : 0u;
     };
     // after the wait that covers their fetch: from here on the registers hold the weights
-    auto landed = [&](u32x4 (&codes)[NTX], u32x2 (&meta)[NTX]) {
+    auto landed = [&](u32x4 (&codes)[NC], u32x2 (&meta)[NTX]) {
 #pragma unroll
-        for (int t = 0; t < NTX; ++t) asm volatile("" : "+v"(codes[t]), "+v"(meta[t]));
+        for (int t = 0; t < NTX; ++t) {
+            if constexpr (Q8)
+                asm volatile("" : "+v"(codes[2 * t]), "+v"(codes[2 * t + 1]), "+v"(meta[t]));
+            else
+                asm volatile("" : "+v"(codes[t]), "+v"(meta[t]));
+        }
     };
-    const NibbleMasks masks = nibble_masks();
+    const NibbleMasks masks = Q8 ? byte_selectors() : nibble_masks();
 
     floatx4 acc[MI][NTW];
     floatx4 acc_shared[XI];
@@ -584,7 +620,7 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     // The matrix instructions are written as asm with the accumulator tied in place (in the
     // accumulation registers); a scheduling barrier after each pins the few vector
     // instructions and the LDS read that follow it in the source to that slot.
-    u32x4 b_codes[3][NTX];
+    u32x4 b_codes[3][NC];
     u32x2 b_meta[3][NTX];
     half2v b_frag[2][NTX][4];  // [set][tile][column pair group]: 8 weights of a lane
     half8 a_frag[MI];
@@ -621,9 +657,9 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     // One quarter: the matrix instructions on b_frag[cur] and the resident fragments; between
     // them the dequantization of quarter next_d (of `codes`) into b_frag[cur ^ 1] and the
     // refill of every fragment, right after its last use, with quarter next_d of next_buffer.
-    auto quarter = [&](auto cur_c, auto next_d_c, uint32_t next_buffer, const u32x4 (&codes)[NTX],
+    auto quarter = [&](auto cur_c, auto next_d_c, uint32_t next_buffer, const u32x4 (&codes)[NC],
                        const u32x2 (&meta)[NTX], auto window_c, uint32_t fetch_buffer,
-                       u32x4 (&fetch_codes)[NTX], u32x2 (&fetch_meta)[NTX]) {
+                       u32x4 (&fetch_codes)[NC], u32x2 (&fetch_meta)[NTX]) {
         constexpr int cur = decltype(cur_c)::value;
         static_for<SLOTS>([&](auto k_c) {
             constexpr int k = decltype(k_c)::value;
@@ -649,8 +685,8 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
                 static_for<3>([&](auto stage_c) {
                     constexpr int stage = decltype(stage_c)::value;
                     if constexpr (Schedule::slot_of(piece, stage) == k)
-                        dequant_stage<stage, piece, decltype(next_d_c)::value>(codes, meta, masks, merged,
-                                                                               centred, b_frag[cur ^ 1]);
+                        dequant_stage<stage, piece, decltype(next_d_c)::value, Q8>(codes, meta, masks, merged,
+                                                                                   centred, b_frag[cur ^ 1]);
                 });
             });
             constexpr int load = Schedule::load_at(decltype(window_c)::value, k);
@@ -685,8 +721,8 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     }
     static_for<PIECES>([&](auto piece_c) {
         static_for<3>([&](auto stage_c) {
-            dequant_stage<decltype(stage_c)::value, decltype(piece_c)::value, 0>(b_codes[0], b_meta[0], masks,
-                                                                                  merged, centred, b_frag[0]);
+            dequant_stage<decltype(stage_c)::value, decltype(piece_c)::value, 0, Q8>(b_codes[0], b_meta[0], masks,
+                                                                                      merged, centred, b_frag[0]);
             asm volatile("s_nop 1");  // packed-fp16 result to its reader: one wait state
         });
     });

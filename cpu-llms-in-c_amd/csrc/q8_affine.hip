@@ -16,6 +16,11 @@
 // read are the Q8 image's plus a second copy of the metadata (+6 %).  The bias sits with the
 // high part so that the GEMM path, which rounds a weight to fp16, rounds the same magnitude
 // the reference's half(scale*q+bias) does.
+//
+// From 17 activation rows on the matrix units would do twice the products that way.  When K is a
+// multiple of 128, prepare therefore also keeps the bytes themselves in GEMM tiles (a second copy
+// of the weight) and the pipelined GEMM kernel multiplies them directly, the weight rounded
+// exactly as half(scale*q+bias); option "q8_gemm" = "doubled" keeps the Q4 kernels.
 #include "device_util.h"
 #include "internal.h"
 
@@ -130,6 +135,90 @@ q8rows_finish_kernel(const float *__restrict__ sum, const float *__restrict__ sc
     store_from_float(y, y_dtype, at, value);
 }
 
+
+// The bytes themselves in GEMM tiles (columns a whole number of 128-column steps): one thread
+// per destination piece of 16 bytes.  Piece (step, tile, half, lane): row 16 * tile + lane % 16,
+// the eight columns 8 * (lane / 16) .. + 7 of quarters 2 * half and 2 * half + 1 of the step, in
+// column order - the matrix instruction's operand layout, two quarters per register.
+// A source row starts row_stride bytes after the one before (only byte aligned: Q8 rows records);
+// flip turns signed bytes into v + 128.
+__global__ void __launch_bounds__(256)
+q8_tiles_kernel(const uint8_t *__restrict__ bytes, size_t row_stride, uint32_t flip, uint32_t N, uint32_t K, uint32_t NT,
+                uint32_t steps, uint4 *__restrict__ tiles)
+{
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (uint64_t)steps * NT * 128u) return;
+    const uint32_t lane = (uint32_t)(index & 63u), half = (uint32_t)(index >> 6) & 1u;
+    const uint64_t record = index >> 7;  // step-major: record = step * NT + tile
+    const uint32_t tile = (uint32_t)(record % NT), step = (uint32_t)(record / NT);
+    const uint32_t row = tile * kTileRows + (lane & 15u), kq = lane >> 4;
+    uint32_t out[4] = {0u, 0u, 0u, 0u};
+    if (row < N) {
+#pragma unroll
+        for (uint32_t q = 0; q < 2; ++q) {
+            const uint32_t column = step * kStepColumns + 32u * (2u * half + q) + 8u * kq;
+            if (column >= K) continue;
+            const uint8_t *source = bytes + (size_t)row * row_stride + column;
+#pragma unroll
+            for (uint32_t c = 0; c < 8; ++c)
+                out[2u * q + c / 4u] |= (uint32_t)(uint8_t)(source[c] ^ flip) << (8u * (c % 4u));
+        }
+    }
+    tiles[index] = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+// Their metadata records: one thread per (step, tile, row), fp16 {scale, bias} of the step's two
+// 64-column groups.  meta_kind < 0: every group of a valid row is {1, -128} (Q8 rows).
+__global__ void __launch_bounds__(256)
+q8_tile_meta_kernel(const uint16_t *__restrict__ meta_a, const uint16_t *__restrict__ meta_b, int meta_kind, uint32_t N,
+                    uint32_t K, uint32_t NT, uint32_t steps, uint2 *__restrict__ out)
+{
+    const uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (uint64_t)steps * NT * 16u) return;
+    const uint32_t r = (uint32_t)(index & 15u);
+    const uint64_t record = index >> 4;
+    const uint32_t tile = (uint32_t)(record % NT), step = (uint32_t)(record / NT);
+    const uint32_t row = tile * kTileRows + r, groups = K / 64u;
+    uint32_t pair[2] = {0u, 0u};
+#pragma unroll
+    for (uint32_t h = 0; h < 2; ++h) {
+        const uint32_t group = 2u * step + h;
+        if (row >= N || group >= groups) continue;
+        const uint64_t block = (uint64_t)row * groups + group;
+        if (meta_kind < 0) {
+            pair[h] = 0x3c00u | 0xd800u << 16;  // fp16 1, fp16 -128
+        } else if (meta_kind == MI355Q_META_F16_INTERLEAVED) {
+            pair[h] = (uint32_t)meta_a[2u * block] | (uint32_t)meta_a[2u * block + 1u] << 16;
+        } else {
+            const _Float16 scale = (_Float16)__builtin_bit_cast(float, (uint32_t)meta_a[block] << 16);
+            const _Float16 bias = (_Float16)__builtin_bit_cast(float, (uint32_t)meta_b[block] << 16);
+            pair[h] = (uint32_t)__builtin_bit_cast(uint16_t, scale) | (uint32_t)__builtin_bit_cast(uint16_t, bias) << 16;
+        }
+    }
+    out[index] = make_uint2(pair[0], pair[1]);
+}
+
+// Allocates and fills the byte tiles of an 8-bit weight (K % 128 == 0); the source is on the device.
+static hipError_t q8_tiles_build(mi355q_context *ctx, const uint8_t *bytes, size_t row_stride, uint32_t flip,
+                                 const uint16_t *meta_a, const uint16_t *meta_b, int meta_kind, uint32_t N, uint32_t K,
+                                 void **allocation, uint4 **codes8, uint2 **meta8)
+{
+    const uint32_t NT = (N + kTileRows - 1u) / kTileRows, steps = K / kStepColumns;
+    const size_t code_bytes = (size_t)steps * NT * 128u * sizeof(uint4), meta_bytes = (size_t)steps * NT * 16u * sizeof(uint2);
+    char *base = nullptr;
+    hipError_t status = hipMalloc((void **)&base, code_bytes + meta_bytes);
+    if (status != hipSuccess) return status;
+    *allocation = base;
+    *codes8 = (uint4 *)base;
+    *meta8 = (uint2 *)(base + code_bytes);
+    const uint64_t pieces = (uint64_t)steps * NT * 128u, records = (uint64_t)steps * NT * 16u;
+    hipLaunchKernelGGL(q8_tiles_kernel, dim3((uint32_t)((pieces + 255u) / 256u)), dim3(256), 0, ctx->stream, bytes,
+                       row_stride, flip, N, K, NT, steps, *codes8);
+    hipLaunchKernelGGL(q8_tile_meta_kernel, dim3((uint32_t)((records + 255u) / 256u)), dim3(256), 0, ctx->stream, meta_a,
+                       meta_b, meta_kind, N, K, NT, steps, *meta8);
+    return hipGetLastError();
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -139,14 +228,16 @@ struct mi355q_q8_weight {
     mi355q_q4_weight *doubled;  // [N][2K]: high-nibble part, then low-nibble part
     uint32_t N, K;
     float *row_scale;  // Q8 rows: the fp32 scale of every output row (device); else null
+    void *byte_tiles;  // the bytes in GEMM tiles and their metadata (doubled->dev.codes8, meta8); null if K % 128
     size_t image_bytes;
 };
 
 extern "C" void mi355q_q8_weight_destroy(mi355q_q8_weight *weight)
 {
     if (weight == nullptr) return;
-    mi355q_q4_weight_destroy(weight->doubled);
+    mi355q_q4_weight_destroy(weight->doubled);  // waits for the stream
     if (weight->row_scale) (void)hipFree(weight->row_scale);
+    if (weight->byte_tiles) (void)hipFree(weight->byte_tiles);
     delete weight;
 }
 
@@ -214,6 +305,12 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
     if (code == MI355Q_OK)  // stream order: the re-tiling kernels run after the split
         code = mi355q_q4_weight_prepare(ctx, scratch + at_codes, scratch + at_m[0], planes ? scratch + at_m[1] : nullptr,
                                         N, 2u * K, meta_kind, MI355Q_SOURCE_DEVICE, &doubled, error, error_capacity);
+    void *byte_tiles = nullptr;
+    if (code == MI355Q_OK && K % kStepColumns == 0u) {
+        status = q8_tiles_build(ctx, (const uint8_t *)d_quants, K, 0u, (const uint16_t *)d_a, (const uint16_t *)d_b, meta_kind,
+                                N, K, &byte_tiles, &doubled->dev.codes8, &doubled->dev.meta8);
+        if (status != hipSuccess) code = fail_hip(status, "q8 byte tiles", error, error_capacity);
+    }
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(scratch);
     mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
@@ -223,6 +320,7 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
     }
     if (code != MI355Q_OK) {
         mi355q_q4_weight_destroy(doubled);
+        if (byte_tiles) (void)hipFree(byte_tiles);
         return code;
     }
     weight->ctx = ctx;
@@ -230,6 +328,7 @@ extern "C" int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants,
     weight->N = N;
     weight->K = K;
     weight->row_scale = nullptr;
+    weight->byte_tiles = byte_tiles;
     weight->image_bytes = code_bytes + groups * 4u;
     *out = weight;
     return MI355Q_OK;
@@ -281,6 +380,12 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
         code = mi355q_q4_weight_prepare(ctx, scratch + at_codes, scratch + at_m[0], scratch + at_m[1], N, 2u * K,
                                         MI355Q_META_BF16_PLANES, MI355Q_SOURCE_DEVICE, &doubled, error,
                                         error_capacity);
+    void *byte_tiles = nullptr;
+    if (code == MI355Q_OK && K % kStepColumns == 0u) {
+        status = q8_tiles_build(ctx, source + 4u, 4u + (size_t)K, 0x80u, nullptr, nullptr, -1, N, K, &byte_tiles,
+                                &doubled->dev.codes8, &doubled->dev.meta8);
+        if (status != hipSuccess) code = fail_hip(status, "q8 rows byte tiles", error, error_capacity);
+    }
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(scratch);
     mi355q_q8_weight *weight = code == MI355Q_OK ? new (std::nothrow) mi355q_q8_weight() : nullptr;
@@ -291,6 +396,7 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
     if (code != MI355Q_OK) {
         mi355q_q4_weight_destroy(doubled);
         if (row_scale) (void)hipFree(row_scale);
+        if (byte_tiles) (void)hipFree(byte_tiles);
         return code;
     }
     weight->ctx = ctx;
@@ -298,6 +404,7 @@ extern "C" int mi355q_q8rows_weight_prepare(mi355q_context *ctx, const void *rec
     weight->N = N;
     weight->K = K;
     weight->row_scale = row_scale;
+    weight->byte_tiles = byte_tiles;
     weight->image_bytes = record_bytes;
     *out = weight;
     return MI355Q_OK;

@@ -133,6 +133,9 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *                                               142-248; tests/qwen38_m3_prefill_parity_test.c:115-199):
  *                                               the launch takes the waves and K slices of the one-row
  *                                               launch instead of the fastest ones for its row count
+ *   "q8_gemm"   = "doubled" / "native"          8-bit weights above 16 rows: the Q4 GEMM kernels on
+ *                                               the doubled weight / the kernel on the bytes
+ *                                               themselves where it applies (the default)
  *   "half_tiles" = "1" / "0"                    the streaming launch's half-tile form (a workgroup takes
  *                                               eight of a tile's rows and two 128-column steps at a
  *                                               time) wherever the kernel has it (up to four 16-bit
@@ -268,8 +271,12 @@ void mi355q_q4_weight_shape(const mi355q_q4_weight *weight, uint32_t *N, uint32_
  * the columns, [high part | low part], which mi355q_q8_linear applies to [x | x] in one Q4
  * linear: the kernels start the activation row over at the weight's second half (K a
  * multiple of 128; otherwise a small kernel first writes the rows twice into a staging
- * buffer); arguments and flags as mi355q_q4_linear.  Small M keeps the weight exact, the GEMM path
- * rounds each part to fp16 as the reference rounds half(scale*q + bias). */
+ * buffer); arguments and flags as mi355q_q4_linear.  Up to 16 rows the weight stays exact.
+ * Above (the GEMM path), when K is a multiple of 128, a kernel multiplies the bytes
+ * themselves, each weight rounded to fp16 as the reference rounds half(scale*q + bias); for
+ * that, prepare keeps the weight a second time in GEMM tiles (device memory: about twice the
+ * image).  Otherwise, and under option "q8_gemm" = "doubled", the Q4 GEMM kernels run on the
+ * doubled weight and round its two parts to fp16 separately. */
 typedef struct mi355q_q8_weight mi355q_q8_weight;
 int mi355q_q8_weight_prepare(mi355q_context *ctx, const void *quants, const void *meta_a,
                              const void *meta_b, uint32_t N, uint32_t K, int meta_kind,

@@ -3,12 +3,16 @@
 Format and reference arithmetic: minimax_h3_q8_gemm_bf16_meta (minimax_h3_attention.metal:594-676),
 u8 quants[N][K], bf16 scales/biases [N][K/64], weight = scale * q + bias.
 Gate for M <= 16 (weights kept exact): max_i |y_i - ref_i| / max(|ref_i|, 1e-2*rms(ref)) <= 1e-3
-against the exact weight with double accumulation.  The GEMM path (M > 16) rounds the two
-nibble halves of a weight to fp16 separately, the reference rounds half(scale*q+bias) once:
-both are within fp16 rounding of the exact weight but not of each other, so the gate there is
-the distance to the exact-weight result, max_i |y_i - ref_i| <= 2e-3 * rms(ref) (the bound the
-Q4 GEMM tests report for fp16-rounded weights), with the reference's own rounding held to the
-same bound for comparison."""
+against the exact weight with double accumulation.  The GEMM path (M > 16) has two forms.  When the
+columns are whole 128-column steps, a kernel multiplies the bytes themselves with the weight rounded
+as the reference rounds it, half(scale*q+bias): gate max_i |y_i - ref_i| <= 1e-5 * rms(ref) against
+the oracle with that rounding (what is left is the order of the fp32 additions and the rare double
+rounding of the reference's fp32 multiply-add).  Otherwise, and under option q8_gemm=doubled, the Q4
+kernels run on the doubled weight and round the two nibble halves of a weight to fp16 separately:
+within fp16 rounding of the exact weight but not of the reference's rounding, so the gate there is the
+distance to the exact-weight result, max_i |y_i - ref_i| <= 2e-3 * rms(ref) (the bound the Q4 GEMM
+tests report for fp16-rounded weights), with the reference's own rounding held to the same bound for
+comparison."""
 import numpy as np
 import pytest
 
@@ -44,7 +48,7 @@ def make_q8(engine, seed, N, K, meta_kind):
                                         (272, 320, 40, "META_BF16_PLANES"),
                                         # long rows, K splits: the activation row starts over inside a split
                                         (560, 2176, 150, "META_BF16_PLANES")])
-def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
+def test_q8_affine_linear(engine, oracle, gpu, force, N, K, M, meta):
     meta_kind = getattr(engine, meta)
     quants, meta_a, meta_b = make_q8(engine, 3, N, K, meta_kind)
     x = np.stack([engine.synth_normal_f32(70 + m, 1.0, K) for m in range(M)]).astype(np.float16)
@@ -56,6 +60,8 @@ def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
         y = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
         y16 = gpu.q8_linear(weight, N, x, engine.F16, engine.F16)
         with_residual = gpu.q8_linear(weight, N, x, engine.F16, engine.F32, residual, engine.F32)
+        force("q8_gemm", "doubled")
+        doubled = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
     finally:
         gpu.q8_destroy(weight)
     exact = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, engine.F16, M)
@@ -69,9 +75,18 @@ def test_q8_affine_linear(engine, oracle, gpu, N, K, M, meta):
         rms = np.sqrt(np.mean(exact * exact, axis=1, keepdims=True))
         ours = float(np.max(np.abs(y - exact) / rms))
         theirs = float(np.max(np.abs(rounded - exact) / rms))
-        print(f"distance to exact weights / rms: this library {ours:.2e}, half(scale*q+bias) {theirs:.2e}", flush=True)
-        assert ours <= 2e-3 and theirs <= 2e-3
+        on_doubled = float(np.max(np.abs(doubled - exact) / rms))
+        to_theirs = float(np.max(np.abs(y - rounded) / rms))
+        print(f"distance to exact weights / rms: this library {ours:.2e} (doubled weight {on_doubled:.2e}), "
+              f"half(scale*q+bias) {theirs:.2e}; this library to half(scale*q+bias) {to_theirs:.2e}", flush=True)
+        assert ours <= 2e-3 and theirs <= 2e-3 and on_doubled <= 2e-3
         assert float(np.max(np.abs(with_residual - (exact + residual)) / rms)) <= 2e-3
+        if K % 128 == 0:  # the kernel on the bytes themselves: the reference's own rounding of a weight
+            assert to_theirs <= 1e-5
+            assert float(np.max(np.abs(y16 - rounded) / rms)) <= 2e-3  # fp16 outputs
+            assert float(np.max(np.abs(with_residual - (rounded + residual)) / rms)) <= 1e-5
+        else:
+            assert np.array_equal(y, doubled)
 
 
 def test_q8rows_f32_against_reference_golden(engine, oracle, gpu):
@@ -136,6 +151,7 @@ def test_q8_affine_under_every_gemm_kernel(engine, oracle, gpu, forced, force):
     """The activation row starts over at the weight's second half of columns in each of the three
     matrix kernels' addressing; every GEMM variant (first kernel, pipelined 16 / 17 / 20 tiles,
     with and without K splits) on a Q8 weight whose doubled row is ten steps long."""
+    force("q8_gemm", "doubled")
     force("q4_gemm", forced)
     N, K, M = 560, 640, 150
     meta_kind = engine.META_BF16_PLANES
@@ -150,3 +166,73 @@ def test_q8_affine_under_every_gemm_kernel(engine, oracle, gpu, forced, force):
     exact = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, x, engine.F16, M)
     rms = np.sqrt(np.mean(exact * exact, axis=1, keepdims=True))
     assert float(np.max(np.abs(y - exact) / rms)) <= 2e-3
+
+
+@pytest.mark.parametrize("x_type", ["F16", "BF16", "F32"])
+@pytest.mark.parametrize("forced", [None, "9,1", "9,2", "9,5"])
+def test_q8_affine_byte_kernel(engine, oracle, gpu, forced, x_type, force):
+    """The GEMM kernel on the bytes themselves, with and without K splits, on a shape with a ragged
+    last block of tiles (35 = 2 x 16 + 3), a ragged last block of rows (150 = 128 + 22) and a
+    number of steps (17) that no split divides; fp16, bf16 and fp32 activations, fp16 metadata,
+    a residual, fp16 and bf16 outputs.  Against the oracle with the reference's rounding of a
+    weight, half(scale*q+bias)."""
+    if forced is not None:
+        force("q4_gemm", forced)
+    N, K, M = 560, 2176, 150
+    meta_kind = engine.META_F16_INTERLEAVED
+    quants, meta_a, meta_b = make_q8(engine, 12, N, K, meta_kind)
+    x32 = np.stack([engine.synth_normal_f32(270 + m, 1.0, K) for m in range(M)])
+    x_dtype = getattr(engine, x_type)
+    if x_type == "F16":
+        x = x32.astype(np.float16)
+        seen = x.astype(np.float32)
+    elif x_type == "BF16":
+        x = bf16_bits(x32)
+        seen = (x.astype(np.uint32) << 16).view(np.float32)
+    else:
+        x = seen = x32
+    residual = engine.synth_normal_f32(98, 1.0, M * N).reshape(M, N)
+    weight = gpu.q8_prepare(quants, meta_a, meta_b, N, K, meta_kind)
+    try:
+        print(f"q8 byte kernel forced={forced} x={x_type}", flush=True)
+        y = gpu.q8_linear(weight, N, x, x_dtype, engine.F32)
+        y16 = gpu.q8_linear(weight, N, x, x_dtype, engine.F16)
+        ybf = gpu.q8_linear(weight, N, x, x_dtype, engine.BF16)
+        with_residual = gpu.q8_linear(weight, N, x, x_dtype, engine.F32, residual, engine.F32)
+    finally:
+        gpu.q8_destroy(weight)
+    rounded = oracle.q8_affine_linear(quants, meta_a, meta_b, meta_kind, N, K, seen, engine.F32, M,
+                                      weight_rounding=oracle.W_ROUND_F16)
+    rms = np.sqrt(np.mean(rounded * rounded, axis=1, keepdims=True))
+    distance = float(np.max(np.abs(y - rounded) / rms))
+    print(f"distance to the oracle with half(scale*q+bias) weights / rms: {distance:.2e}", flush=True)
+    # fp16 and bf16 activations enter the matrix units exactly (bf16 after a power-of-two scaling of the
+    # row); fp32 ones as fp16 value + remainder, 2^-22 relative per element
+    assert distance <= 1e-5
+    assert float(np.max(np.abs(with_residual - (rounded + residual)) / rms)) <= 1e-5
+    assert float(np.max(np.abs(y16.astype(np.float64) - rounded) / rms)) <= 2e-3
+    bf = (ybf.astype(np.uint32) << 16).view(np.float32) if ybf.dtype == np.uint16 else ybf
+    assert float(np.max(np.abs(bf.astype(np.float64) - rounded) / rms)) <= 1.6e-2
+
+
+def test_q8rows_byte_kernel_matches_doubled_weight(engine, oracle, gpu, force):
+    """Q8 rows on the GEMM path: integer weights v = byte - 128 are exact in fp16 in both forms (the
+    bytes themselves with {1, -128}; the nibble halves with {16, -128} and {1, 0}), so the two forms
+    differ only in the order of the fp32 additions."""
+    N, K, M = 400, 1280, 72
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    rows = oracle.q8_weight_quantize(w)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    weight = gpu.q8rows_prepare(rows, N, K)
+    try:
+        print("q8 rows, byte kernel and doubled weight", flush=True)
+        native = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
+        force("q8_gemm", "doubled")
+        doubled = gpu.q8_linear(weight, N, x, engine.F16, engine.F32)
+    finally:
+        gpu.q8_destroy(weight)
+    ref = oracle.q8rows_f32_linear(rows, N, K, x.astype(np.float32)).astype(np.float64)
+    rms = np.sqrt(np.mean(ref * ref, axis=1, keepdims=True))
+    assert float(np.max(np.abs(native - ref) / rms)) <= 5e-5
+    assert float(np.max(np.abs(doubled - ref) / rms)) <= 5e-5
