@@ -91,6 +91,11 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "gemm_order") == 0) {  // "xcd" / "launch"
+        if (set && strcmp(value, "xcd") != 0 && strcmp(value, "launch") != 0) return MI355Q_ERROR_INVALID;
+        ctx->gemm_order = !set ? -1 : strcmp(value, "xcd") == 0 ? 1 : 0;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "q8_gemm") == 0) {  // "doubled": no 8-bit GEMM kernel; "native" or unset: use it where it applies
         if (set && strcmp(value, "doubled") != 0 && strcmp(value, "native") != 0) return MI355Q_ERROR_INVALID;
         ctx->q8_gemm_doubled = set && strcmp(value, "doubled") == 0;
@@ -183,6 +188,7 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
         return MI355Q_ERROR_RUNTIME;
     }
     memset(ctx, 0, sizeof *ctx);
+    ctx->gemm_order = -1;
     ctx->device = device;
     ctx->profile_events = new (std::nothrow) std::vector<hipEvent_t>();
     hipError_t status = ctx->profile_events ? hipSuccess : hipErrorOutOfMemory;

@@ -28,6 +28,7 @@ struct GemmParams {
     int y_dtype, residual_dtype;
     int residual_is_bias;  // residual is one row [N], added to every activation row
     int wide_stores;       // N % 4 == 0 and y 16-byte aligned: four adjacent outputs go out as one store
+    int xcd_order;         // pipelined kernel: blocks that share weights are placed on one XCD (see there)
 };
 
 __device__ __forceinline__ half8 dequant8(uint32_t word, const NibbleMasks &masks, half8 scale,
@@ -508,11 +509,25 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15u;
     const uint32_t kq = lane >> 4;
-    const uint32_t m0 = blockIdx.y * BM;
-    const uint32_t block_first_tile = blockIdx.x * TPB;
+    // Which block of the problem this workgroup takes.  Workgroups go to the eight XCDs in turn
+    // (workgroup L of the launch to XCD L % 8), and the row blocks that multiply the same weights
+    // should meet in one XCD's L2: with xcd_order, XCD i works through a contiguous run of the
+    // problem's blocks numbered row block fastest, then tile block, then K split.
+    uint32_t block_n = blockIdx.x, block_m = blockIdx.y, split = blockIdx.z;
+    if (p.xcd_order) {
+        const uint32_t total = gridDim.x * gridDim.y * gridDim.z;
+        const uint32_t launch_index = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const uint32_t xcd = launch_index % 8u, base = total / 8u, longer = total % 8u;  // XCDs 0 .. longer-1 get base + 1
+        const uint32_t first = xcd < longer ? xcd * (base + 1u) : longer * (base + 1u) + (xcd - longer) * base;
+        const uint32_t number = first + launch_index / 8u;
+        block_m = number % gridDim.y;
+        block_n = number / gridDim.y % gridDim.x;
+        split = number / (gridDim.y * gridDim.x);
+    }
+    const uint32_t m0 = block_m * BM;
+    const uint32_t block_first_tile = block_n * TPB;
     const uint32_t tile0 = block_first_tile + wave * NTW;
     const uint32_t shared_tile = block_first_tile + 4u * NTW;
-    const uint32_t split = blockIdx.z;
     const uint32_t step_begin = split * p.steps_per_split;
     const uint32_t step_end = step_begin + p.steps_per_split < p.T ? step_begin + p.steps_per_split : p.T;
     if (step_begin >= step_end) return;  // uniform over the workgroup

@@ -133,6 +133,9 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *                                               142-248; tests/qwen38_m3_prefill_parity_test.c:115-199):
  *                                               the launch takes the waves and K slices of the one-row
  *                                               launch instead of the fastest ones for its row count
+ *   "gemm_order" = "xcd" / "launch"             the pipelined GEMM numbers its blocks so that the row
+ *                                               blocks of one tile block share an XCD's L2 / takes them
+ *                                               in launch order; unset: by the number of tile blocks
  *   "q8_gemm"   = "doubled" / "native"          8-bit weights above 16 rows: the Q4 GEMM kernels on
  *                                               the doubled weight / the kernel on the bytes
  *                                               themselves where it applies (the default)

@@ -232,3 +232,27 @@ def test_hand_scheduled_loads_match_compiler_managed_loads(engine, gpu, force, N
     assert np.array_equal(scheduled.view(np.uint32), plain.view(np.uint32))
     assert np.any(scheduled != 0)
 
+
+
+@pytest.mark.parametrize("N,K,M,forced", [(1104, 2176, 400, "6,2"), (1104, 2176, 150, "7,3"), (5120, 640, 300, "8,1"),
+                                          (560, 384, 70, "6,1")])
+def test_block_order_does_not_change_the_bits(engine, gpu, force, N, K, M, forced):
+    """The pipelined kernel either takes its blocks in launch order or renumbers them so that the
+    row blocks of one tile block run on one XCD (numbers of blocks that are and are not multiples
+    of eight, with K splits, ragged last blocks): every block is computed exactly once either way,
+    so the outputs are the same bits."""
+    kind = engine.META_BF16_PLANES
+    quants, meta_a, meta_b = engine.synth_q4_affine(71, 0.02, N, K, kind)
+    x = make_x(engine, 72, M, K).astype(np.float16)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, kind)
+    try:
+        force("q4_gemm", forced)
+        print(f"gemm block order N={N} K={K} M={M} forced={forced}", flush=True)
+        force("gemm_order", "launch")
+        in_launch_order = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+        force("gemm_order", "xcd")
+        renumbered = gpu.q4_linear(weight, x, engine.F16, engine.F32)
+    finally:
+        weight.destroy()
+    assert np.array_equal(in_launch_order.view(np.uint32), renumbered.view(np.uint32))
+    assert np.any(renumbered != 0)
