@@ -257,6 +257,9 @@ static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const
     case 20202: return launch_one<MP, 2, 2, 2>(ctx, p);
     case 20204: return launch_one<MP, 2, 2, 4>(ctx, p);
     case 20208: return launch_one<MP, 2, 2, 8>(ctx, p);
+    case 30204:
+        if constexpr (MP >= 4) return launch_one<MP, 3, 2, 4>(ctx, p);
+        break;
     case 40202: return launch_one<MP, 4, 2, 2>(ctx, p);
     case 40204: return launch_one<MP, 4, 2, 4>(ctx, p);
     case 40208: return launch_one<MP, 4, 2, 8>(ctx, p);
@@ -289,6 +292,8 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         shape = choose_shape(ctx, NT_total, T, 1, fused);
         shape.mp = mp;
         shape.tb = mp >= 4 && NT_total >= cus ? 2 : mp >= 4 ? 1 : shape.tb;
+        if (mp >= 4 && !fused && shape.waves == 4 && NT_total > 8u * cus && (NT_total + 2u) / 3u <= 4u * cus)
+            shape.tb = 3;  // one round of workgroups instead of one and a few (see below)
         while (shape.tb > 1 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u) shape.tb /= 2;
         return shape;
     }
@@ -325,6 +330,14 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         // slices (of 32 steps or more: adding the slices costs about as much as a few
         // steps) until some two workgroups per compute unit exist.
         shape.tb = NT_total >= cus ? 2 : 1;
+        // These kernels hold four workgroups of four waves per compute unit (104-126 registers).
+        // When the pairs of tiles are a few more than that (gate|up: 1088 on 1024 places), the ones
+        // left over start when the others end and run alone at the pace of their own chain of
+        // round trips (3 us of a 21-25 us launch); three tiles per workgroup fit in one round and
+        // share a step's activations three ways (gate|up at M = 4 / 8 / 16: 21.8 -> 20.8,
+        // 24.8 -> 22.2, 35.2 -> 27.4 us; four tiles: 25.4 / 26.4 / 32.6).  A fused pair takes
+        // equal numbers of gate and up tiles and stays with two.
+        if (!fused && NT_total > 8u * cus && (NT_total + 2u) / 3u <= 4u * cus) shape.tb = 3;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
         slices = 2u * cus / groups;
         if (slices > T / 32u) slices = T / 32u;

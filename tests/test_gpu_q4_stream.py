@@ -572,3 +572,58 @@ def test_half_tile_form(engine, oracle, gpu, force, name, rows, K, M, x_dtype, w
         assert q4_relative_error(results["1"][i], reference) <= TOLERANCE
         assert q4_relative_error(results["0"][i], reference) <= TOLERANCE
         assert np.array_equal(results["1"][i].view(np.uint32), results["1 again"][i].view(np.uint32))
+
+
+THREE_TILE_CASES = [
+    # name, rows of the targets, K, M, x dtype, residual, forced launch shape
+    ("gate_up_sized_m8", (17408, 17408), 640, 8, "F16", False, None),   # chosen by the library itself: 2176 tiles
+    ("ragged_tiles_m4", (1000, 520), 1024, 4, "F16", True, "3,2,4"),    # 63 and 33 tiles: last workgroups of one and two tiles
+    ("bf16_rows_m16", (1000,), 704, 16, "BF16", False, "3,2,4"),        # sixteen rows, odd number of 64-column groups
+    ("fp32_rows_m5", (808, 808, 200), 1536, 5, "F32", True, "3,2,4"),   # ten operand rows (value, remainder)
+    ("k_slices_m8", (600,), 4096, 8, "F16", False, "3,2,4,2"),          # two K slices added inside the kernel
+]
+
+
+@pytest.mark.parametrize("name,rows,K,M,x_dtype,with_residual,forced", THREE_TILE_CASES,
+                         ids=[c[0] for c in THREE_TILE_CASES])
+def test_three_tiles_per_workgroup(engine, oracle, gpu, force, name, rows, K, M, x_dtype, with_residual, forced):
+    """Three tiles per workgroup (what gate|up of the 27B layer takes from four rows on, so that its
+    workgroups fit the compute units in one round): against the oracle, and bit for bit against the
+    launch with two tiles per workgroup (tiles do not meet: which workgroup computes a tile cannot
+    change its sums)."""
+    x_dtype = getattr(engine, x_dtype)
+    kind = engine.META_BF16_PLANES
+    images = [engine.synth_q4_affine(500 + i, 0.02, N, K, kind) for i, N in enumerate(rows)]
+    weights = [gpu.q4_prepare(*image, N, K, kind) for image, N in zip(images, rows)]
+    x = make_x(engine, 510, M, K, x_dtype)
+    residuals = [engine.synth_normal_f32(520 + i, 1.0, M * N).reshape(M, N) if with_residual else None
+                 for i, N in enumerate(rows)]
+    pointers = []
+    try:
+        print(f"three tile case {name}", flush=True)
+        x_ptr = gpu.to_device(x)
+        y_ptrs = [gpu.alloc(M * N * 4) for N in rows]
+        r_ptrs = [gpu.to_device(r) if r is not None else None for r in residuals]
+        pointers = [x_ptr] + y_ptrs + [p for p in r_ptrs if p]
+        calls = engine.make_calls([([(w, y, r) for w, y, r in zip(weights, y_ptrs, r_ptrs)], x_ptr, x_dtype, M,
+                                    engine.F32, engine.F32)])
+        results = {}
+        two = "2,2,4" + (forced[5:] if forced and len(forced) > 5 else "")
+        for mode, shape in (("three", forced), ("two", two)):
+            force("q4_stream", shape)
+            for y_ptr, N in zip(y_ptrs, rows):
+                gpu.upload(y_ptr, np.full((M, N), np.nan, dtype=np.float32))
+            gpu.q4_sequence(calls)
+            gpu.sync()
+            results[mode] = [gpu.download(y_ptr, (M, N), np.float32) for y_ptr, N in zip(y_ptrs, rows)]
+    finally:
+        for pointer in pointers:
+            gpu.free(pointer)
+        for weight in weights:
+            weight.destroy()
+    for i, N in enumerate(rows):
+        reference = oracle.q4_linear(*images[i], kind, N, K, x, x_dtype, M)
+        if with_residual:
+            reference = reference + residuals[i]
+        assert q4_relative_error(results["three"][i], reference) <= TOLERANCE
+        assert np.array_equal(results["three"][i].view(np.uint32), results["two"][i].view(np.uint32))
