@@ -91,6 +91,10 @@ static int apply_option(mi355q_context *ctx, const char *name, const char *value
         ctx->gemm_plain_loads = set;
         return MI355Q_OK;
     }
+    if (strcmp(name, "three_tiles") == 0) {  // "0": never; unset: by shape
+        ctx->three_tiles = set && strcmp(value, "0") == 0 ? 0 : -1;
+        return MI355Q_OK;
+    }
     if (strcmp(name, "gemm_order") == 0) {  // "xcd" / "launch"
         if (set && strcmp(value, "xcd") != 0 && strcmp(value, "launch") != 0) return MI355Q_ERROR_INVALID;
         ctx->gemm_order = !set ? -1 : strcmp(value, "xcd") == 0 ? 1 : 0;
@@ -189,6 +193,7 @@ int mi355q_context_create(int device, mi355q_context **out, char *error,
     }
     memset(ctx, 0, sizeof *ctx);
     ctx->gemm_order = -1;
+    ctx->three_tiles = -1;
     ctx->device = device;
     ctx->profile_events = new (std::nothrow) std::vector<hipEvent_t>();
     hipError_t status = ctx->profile_events ? hipSuccess : hipErrorOutOfMemory;

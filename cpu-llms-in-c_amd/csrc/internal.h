@@ -90,6 +90,7 @@ struct mi355q_context {
     // waves and K slices of the one-row launch, so that a row's result does not depend on the batch
     bool batch_invariant;
     int half_tiles;  // option "half_tiles": -1 the launch decides, 1 wherever the kernel can, 0 never
+    int three_tiles;        // option "three_tiles" = "0": the streaming launch never takes three tiles per workgroup (-1: by shape)
     int gemm_order;         // option "gemm_order": 1 = "xcd" (the pipelined GEMM places blocks that share weights on one XCD), 0 = "launch", -1 = by shape
     bool q8_gemm_doubled;   // option "q8_gemm" = "doubled": 8-bit weights take the Q4 GEMM kernels on their doubled form
     bool gemm_plain_loads;  // option "gemm_loads" = "plain": the 17-tile GEMM shape with compiler-managed weight loads

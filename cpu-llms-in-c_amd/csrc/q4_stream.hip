@@ -257,9 +257,7 @@ static hipError_t launch_shape(mi355q_context *ctx, const StreamParams &p, const
     case 20202: return launch_one<MP, 2, 2, 2>(ctx, p);
     case 20204: return launch_one<MP, 2, 2, 4>(ctx, p);
     case 20208: return launch_one<MP, 2, 2, 8>(ctx, p);
-    case 30204:
-        if constexpr (MP >= 4) return launch_one<MP, 3, 2, 4>(ctx, p);
-        break;
+    case 30204: return launch_one<MP, 3, 2, 4>(ctx, p);
     case 40202: return launch_one<MP, 4, 2, 2>(ctx, p);
     case 40204: return launch_one<MP, 4, 2, 4>(ctx, p);
     case 40208: return launch_one<MP, 4, 2, 8>(ctx, p);
@@ -277,6 +275,15 @@ static void choose_cuts(StreamShape &shape, uint32_t T, uint32_t slices)
     shape.slices = (T + shape.slice_steps - 1) / shape.slice_steps;
 }
 
+// More tiles than workgroups of one or two tiles find places at once (eight of four waves per
+// compute unit at best), and few enough that workgroups of three tiles run in one round (four per
+// compute unit).  A fused pair takes equal numbers of gate and up tiles: never three.
+static bool three_tiles_fit(const mi355q_context *ctx, uint32_t NT_total, bool fused)
+{
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    return ctx->three_tiles != 0 && !fused && NT_total > 8u * cus && (NT_total + 2u) / 3u <= 4u * cus;
+}
+
 StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t T, int mp, bool fused)
 {
     StreamShape shape;
@@ -292,7 +299,7 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         shape = choose_shape(ctx, NT_total, T, 1, fused);
         shape.mp = mp;
         shape.tb = mp >= 4 && NT_total >= cus ? 2 : mp >= 4 ? 1 : shape.tb;
-        if (mp >= 4 && !fused && shape.waves == 4 && NT_total > 8u * cus && (NT_total + 2u) / 3u <= 4u * cus)
+        if (mp >= 4 && shape.waves == 4 && three_tiles_fit(ctx, NT_total, fused))
             shape.tb = 3;  // one round of workgroups instead of one and a few (see below)
         while (shape.tb > 1 && stream_lds_bytes(mp, shape.tb, shape.depth, shape.waves) + 64u > 64u * 1024u) shape.tb /= 2;
         return shape;
@@ -310,8 +317,17 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         // the tiles are few (q|k|v 7.3 against 8.15 us with four).  Only a matrix with tens of
         // thousands of tiles (the LM head) takes two or four per workgroup, two waves each.
         shape.tb = NT_total >= 32u * cus ? 4 : NT_total >= 12u * cus ? 2 : 1;
-        const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
+        uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
         shape.waves = shape.tb > 1 ? 2 : groups <= 3u * cus ? 8 : 4;
+        // A few more tiles than the compute units hold workgroups at once (gate|up: 2176 on 2048
+        // places at one row, 1792 at two): three tiles per workgroup of four waves make it one
+        // round of 726 (124-126 registers: four workgroups per compute unit); gate|up 18.8-19.6
+        // -> 18.2-18.5 us at one row, 19.5-20.0 -> 18.5-18.8 at two (pairs of tiles: 19.2 / 22.0)
+        if (three_tiles_fit(ctx, NT_total, fused)) {
+            shape.tb = 3;
+            shape.waves = 4;
+            groups = (NT_total + 2u) / 3u;
+        }
         // one row and two workgroups per compute unit (q|k|v: 512 tiles of 40 steps): sixteen
         // waves put nearly the whole matrix in flight at once, 6.8-6.9 against 7.2-7.4 us
         // (with two rows, or 320 tiles, eight are better)
@@ -337,7 +353,7 @@ StreamShape choose_shape(const mi355q_context *ctx, uint32_t NT_total, uint32_t 
         // share a step's activations three ways (gate|up at M = 4 / 8 / 16: 21.8 -> 20.8,
         // 24.8 -> 22.2, 35.2 -> 27.4 us; four tiles: 25.4 / 26.4 / 32.6).  A fused pair takes
         // equal numbers of gate and up tiles and stays with two.
-        if (!fused && NT_total > 8u * cus && (NT_total + 2u) / 3u <= 4u * cus) shape.tb = 3;
+        if (three_tiles_fit(ctx, NT_total, fused)) shape.tb = 3;
         const uint32_t groups = (NT_total + shape.tb - 1) / (uint32_t)shape.tb;
         slices = 2u * cus / groups;
         if (slices > T / 32u) slices = T / 32u;

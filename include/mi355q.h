@@ -133,6 +133,8 @@ int mi355q_context_info(mi355q_context *ctx, mi355q_device_info *info,
  *                                               142-248; tests/qwen38_m3_prefill_parity_test.c:115-199):
  *                                               the launch takes the waves and K slices of the one-row
  *                                               launch instead of the fastest ones for its row count
+ *   "three_tiles" = "0"                         the streaming launch never takes three tiles per
+ *                                               workgroup (unset: where two would not fit one round)
  *   "gemm_order" = "xcd" / "launch"             the pipelined GEMM numbers its blocks so that the row
  *                                               blocks of one tile block share an XCD's L2 / takes them
  *                                               in launch order; unset: by the number of tile blocks
