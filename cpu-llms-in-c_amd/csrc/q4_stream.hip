@@ -24,7 +24,7 @@
 // Long rows of matrices with few tiles are cut in slices over workgroups (fp32
 // partial sums, added in slice order by whichever workgroup of the column
 // finishes last).
-#include "q4_stream_device.h"
+#include "q4_stream_kernels.h"
 #include "q4_stream_host.h"
 
 #include <cstdio>
@@ -74,20 +74,15 @@ __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t *words, uint32
     if (index < count) words[index] = 0u;
 }
 
-template <int MP, int TB, int D, int W, bool BF, bool WRAP = false>
-__global__ void __launch_bounds__(64 * W) q4_stream_kernel(const StreamParams p)
-{
-    extern __shared__ uint4 lds[];
-    stream_workgroup<MP, TB, D, W, BF, WRAP, kStreamPlain>(p, ChainParams{}, blockIdx.x, blockIdx.y, lds);
-}
-
-// The half-tile form (see stream_workgroup): MP operand rows = two per activation row.
-template <int MP, int W, bool BF>
-__global__ void __launch_bounds__(64 * W) q4_stream_half_kernel(const StreamParams p)
-{
-    extern __shared__ uint4 lds[];
-    stream_workgroup<MP, 1, 2, W, BF, false, kStreamPlain, true>(p, ChainParams{}, blockIdx.x, 0u, lds);
-}
+// the kernels are compiled in q4_stream_rows_*.hip
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DECLARE, 1)
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DECLARE, 2)
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DECLARE, 4)
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DECLARE, 8)
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DECLARE, 16)
+MI355Q_STREAM_SHAPES_SIXTEEN_WAVES(MI355Q_STREAM_DECLARE, 1)
+MI355Q_STREAM_SHAPES_SIXTEEN_WAVES(MI355Q_STREAM_DECLARE, 2)
+MI355Q_STREAM_HALF_SHAPES(MI355Q_STREAM_HALF_DECLARE)
 
 // Adds the slices' partial sums in slice order (a fixed order) and applies the
 // epilogue.  One thread per output element of all targets.

@@ -1,0 +1,8 @@
+// The streaming kernels for three and four activation rows (a file per row count: they compile side by side).
+#include "q4_stream_kernels.h"
+
+namespace mi355q {
+
+MI355Q_STREAM_SHAPES(MI355Q_STREAM_DEFINE, 4)
+
+}  // namespace mi355q
