@@ -566,8 +566,8 @@ def measure_q8_affine(engine, ctx, rows_list=(1, 256), copies=3):
             entry.update({"tflops": round(achieved, 1),
                           "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": F16_MFMA_PEAK_TFLOPS,
                                        "unit": "TFLOP/s", "frac": round(achieved / F16_MFMA_PEAK_TFLOPS, 4),
-                                       "kernel": "q4_gemm_pipe_kernel<128, 4, false, false, true>: 8-bit codes, "
-                                                 "16 tiles per workgroup"}})
+                                       "kernel": "q4_gemm_pipe_kernel<128, 3, true, false, true>: 8-bit codes, "
+                                                 "13 tiles per workgroup (16 where they fill the compute units better)"}})
         out["q8_affine_g64_m%d" % M] = entry
         ctx.free(x_ptr)
         ctx.free(y_ptr)

@@ -41,6 +41,7 @@ extern template __global__ void q4_gemm_pipe_kernel<128, 4, true, false>(const G
 extern template __global__ void q4_gemm_pipe_kernel<128, 4, true, true>(const GemmParams);
 extern template __global__ void q4_gemm_pipe_kernel<128, 5, false, false>(const GemmParams);
 extern template __global__ void q4_gemm_pipe_kernel<128, 4, false, false, true>(const GemmParams);  // 8-bit codes
+extern template __global__ void q4_gemm_pipe_kernel<128, 3, true, false, true>(const GemmParams);   // 8-bit codes
 
 // Adds the K splits in split order (a fixed order) and applies the epilogue.  WIDE: a thread
 // takes four adjacent outputs of one row (N a multiple of 4, y 16-byte aligned): 16-byte loads
@@ -128,18 +129,19 @@ static hipError_t launch_pipe(mi355q_context *ctx, dim3 grid, const GemmParams &
     return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT>, grid, dim3(256), bytes, p);
 }
 
-// The 16-tile shape on 8-bit codes.
+// The shapes on 8-bit codes: 16 tiles, or 13 (three per wave and one shared).
+template <int NTW, bool XT>
 static hipError_t launch_pipe_bytes(mi355q_context *ctx, dim3 grid, const GemmParams &p)
 {
     constexpr size_t bytes = pipe_lds_bytes(128);
-    constexpr int slot = 14;
+    constexpr int slot = XT ? 13 : 14;
     if (!ctx->lds_raised[slot]) {
-        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, 4, false, false, true>,
+        hipError_t status = hipFuncSetAttribute((const void *)q4_gemm_pipe_kernel<128, NTW, XT, false, true>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (status != hipSuccess) return status;
         ctx->lds_raised[slot] = true;
     }
-    return launch(ctx, q4_gemm_pipe_kernel<128, 4, false, false, true>, grid, dim3(256), bytes, p);
+    return launch(ctx, q4_gemm_pipe_kernel<128, NTW, XT, false, true>, grid, dim3(256), bytes, p);
 }
 
 // The 17-tile shape with compiler-managed weight loads (option "gemm_loads" = "plain").
@@ -231,8 +233,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
         {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
         {128, 4, 0, 1, 0.0, 0.0, 1.493}, {128, 4, 1, 1, 0.0, 0.0, 1.675}, {128, 5, 0, 1, 0.0, 0.0, 1.849},
-        {128, 4, 0, 1, 0.0, 0.0, 1.60}};  // 9: the 16-tile shape on 8-bit codes, and only for them
-    constexpr int kBytesVariant = 9;
+        {128, 4, 0, 1, 0.0, 0.0, 1.60}, {128, 3, 1, 1, 0.0, 0.0, 1.33}};  // 9, 10: 16 and 13 tiles on 8-bit codes, and only for them
+    constexpr int kBytesVariant = 9;  // the first of them
     // A round of the pipelined kernel that fills only the fraction r of the compute units runs
     // faster than a full one: the chip is power limited, and up to about half of it the clock
     // stays near its maximum, from there it falls to the sustained clock of a full chip
@@ -250,7 +252,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     const bool pipe_ok = w.K % kStepColumns == 0 && (uint64_t)rows * x_columns * sizeof(_Float16) + 16384u < (1ull << 32);
     for (int v = 0; v < (int)(sizeof variants / sizeof variants[0]); ++v) {
         if (v >= 6 && !pipe_ok) continue;
-        if ((v == kBytesVariant) != bytes_native) continue;
+        if ((v >= kBytesVariant) != bytes_native) continue;
         const Variant &c = variants[v];
         const uint32_t tpb = 4u * c.ntw + c.extra;
         const uint32_t slots = cus * (uint32_t)c.resident;
@@ -294,7 +296,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     }
     // option "q4_gemm" = "VARIANT,SPLITS" for experiments
     if (ctx->force_gemm[1] >= 1 && ctx->force_gemm[0] < (int)(sizeof variants / sizeof variants[0]) &&
-        (ctx->force_gemm[0] < 6 || pipe_ok) && (ctx->force_gemm[0] == kBytesVariant) == bytes_native) {
+        (ctx->force_gemm[0] < 6 || pipe_ok) && (ctx->force_gemm[0] >= kBytesVariant) == bytes_native) {
         best = ctx->force_gemm[0];
         best_splits = (uint32_t)ctx->force_gemm[1];
     }
@@ -336,7 +338,8 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
     case 6: launched = launch_pipe<4, false>(ctx, grid, p); break;
     case 7: launched = ctx->gemm_plain_loads ? launch_pipe_plain(ctx, grid, p) : launch_pipe<4, true>(ctx, grid, p); break;
     case 8: launched = launch_pipe<5, false>(ctx, grid, p); break;
-    default: launched = launch_pipe_bytes(ctx, grid, p); break;
+    case 9: launched = launch_pipe_bytes<4, false>(ctx, grid, p); break;
+    default: launched = launch_pipe_bytes<3, true>(ctx, grid, p); break;
     }
     if (launched != hipSuccess)
         return fail_hip(launched, "q4 gemm kernel launch", error, error_capacity);

@@ -786,8 +786,10 @@ __global__ void __launch_bounds__(256, 1) q4_gemm_pipe_kernel(const GemmParams p
         else asm volatile("s_nop 15\n\ts_nop 15");
 #pragma unroll
         for (int i = MI - 1; i >= 0; --i) {
-            static_assert(NTW == 4 || NTW == 5, "the accumulators of one row group in one statement");
-            if constexpr (NTW == 4)
+            static_assert(NTW == 3 || NTW == 4 || NTW == 5, "the accumulators of one row group in one statement");
+            if constexpr (NTW == 3)
+                asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]));
+            else if constexpr (NTW == 4)
                 asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]));
             else
                 asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][NTW - 1]));

@@ -169,7 +169,7 @@ def test_q8_affine_under_every_gemm_kernel(engine, oracle, gpu, forced, force):
 
 
 @pytest.mark.parametrize("x_type", ["F16", "BF16", "F32"])
-@pytest.mark.parametrize("forced", [None, "9,1", "9,2", "9,5"])
+@pytest.mark.parametrize("forced", [None, "9,1", "9,2", "9,5", "10,1", "10,3"])
 def test_q8_affine_byte_kernel(engine, oracle, gpu, forced, x_type, force):
     """The GEMM kernel on the bytes themselves, with and without K splits, on a shape with a ragged
     last block of tiles (35 = 2 x 16 + 3), a ragged last block of rows (150 = 128 + 22) and a
