@@ -233,7 +233,7 @@ int q4_gemm_linear(mi355q_context *ctx, const Q4LinearArgs &a, uint32_t target, 
         {128, 4, 0, 2, 0.399, 0.491, 0.0}, {128, 2, 0, 2, 0.327, 0.434, 0.0}, {64, 4, 0, 3, 0.333, 0.460, 0.0},
         {64, 4, 1, 2, 0.347, 0.444, 0.0},  {64, 2, 0, 4, 0.288, 0.422, 0.0},  {64, 2, 1, 2, 0.308, 0.443, 0.0},
         {128, 4, 0, 1, 0.0, 0.0, 1.493}, {128, 4, 1, 1, 0.0, 0.0, 1.675}, {128, 5, 0, 1, 0.0, 0.0, 1.849},
-        {128, 4, 0, 1, 0.0, 0.0, 1.60}, {128, 3, 1, 1, 0.0, 0.0, 1.33}};  // 9, 10: 16 and 13 tiles on 8-bit codes, and only for them
+        {128, 4, 0, 1, 0.0, 0.0, 1.60}, {128, 3, 1, 1, 0.0, 0.0, 1.40}};  // 9, 10: 16 and 13 tiles on 8-bit codes, and only for them
     constexpr int kBytesVariant = 9;  // the first of them
     // A round of the pipelined kernel that fills only the fraction r of the compute units runs
     // faster than a full one: the chip is power limited, and up to about half of it the clock
