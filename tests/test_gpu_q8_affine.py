@@ -47,7 +47,9 @@ def make_q8(engine, seed, N, K, meta_kind):
                                         # K not a whole number of 128-column steps: the rows are written twice first
                                         (272, 320, 40, "META_BF16_PLANES"),
                                         # long rows, K splits: the activation row starts over inside a split
-                                        (560, 2176, 150, "META_BF16_PLANES")])
+                                        (560, 2176, 150, "META_BF16_PLANES"),
+                                        # one tile and one step; a ragged second tile under many row blocks
+                                        (16, 128, 17, "META_F16_INTERLEAVED"), (17, 256, 1000, "META_BF16_PLANES")])
 def test_q8_affine_linear(engine, oracle, gpu, force, N, K, M, meta):
     meta_kind = getattr(engine, meta)
     quants, meta_a, meta_b = make_q8(engine, 3, N, K, meta_kind)
