@@ -323,6 +323,36 @@ def test_row_subsets(engine, oracle, gpu, M, x_dtype, meta_kind):
     assert q4_relative_error(gathered, full[:, ids].astype(np.float64)) <= 1e-4
 
 
+@pytest.mark.parametrize("M", [1, 4])
+def test_row_subsets_with_three_tiles_per_workgroup(engine, oracle, gpu, force, M):
+    """A prefix and a gathered list of rows under the three-tile launch shape (what a restricted
+    vocabulary of 33 to 49 thousand rows takes): the same values as the library's own shape for
+    these small subsets, bit for bit (which workgroup computes a tile does not change its sums
+    as long as the waves and K slices are the same), and the oracle's to the tolerance."""
+    kind = engine.META_BF16_PLANES
+    N, K = 1000, 1536
+    quants, meta_a, meta_b = engine.synth_q4_affine(34, 0.02, N, K, kind)
+    x = make_x(engine, 35, M, K, engine.F16)
+    rng = np.random.default_rng(36)
+    ids = np.concatenate([[N - 1, 0, 17, 17], rng.integers(0, N, size=90)]).astype(np.uint32)
+    weight = gpu.q4_prepare(quants, meta_a, meta_b, N, K, kind)
+    try:
+        print(f"row subsets, three tiles per workgroup, M={M}", flush=True)
+        results = {}
+        for shape in ("3,2,4", "1,2,4"):
+            force("q4_stream", shape)
+            results[shape] = (gpu.q4_linear_rows(weight, None, x, engine.F16, engine.F32, count=203),
+                              gpu.q4_linear_rows(weight, ids, x, engine.F16, engine.F32))
+    finally:
+        weight.destroy()
+    ref = oracle.q4_linear(quants, meta_a, meta_b, kind, N, K, x, engine.F16, M)
+    prefix, gathered = results["3,2,4"]
+    assert q4_relative_error(prefix, ref[:, :203]) <= TOLERANCE
+    assert q4_relative_error(gathered, ref[:, ids]) <= TOLERANCE
+    assert np.array_equal(prefix.view(np.uint32), results["1,2,4"][0].view(np.uint32))
+    assert np.array_equal(gathered.view(np.uint32), results["1,2,4"][1].view(np.uint32))
+
+
 def test_row_subset_with_device_ids(engine, oracle, gpu):
     """Row ids that already live on the GPU (MI355Q_SOURCE_DEVICE, asynchronous call): an id past
     the matrix yields 0 instead of being refused, the rest equals the host-id call bit for bit."""
